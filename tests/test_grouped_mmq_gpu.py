@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import QTYPES, assert_matches_f32_reference, bits, f32, nrmse, random_bf16
+from helpers import QTYPES, assert_matches_f32_reference, bits, f32, max_rel_to_peak, nrmse, random_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -51,6 +51,7 @@ def test_grouped_forward_matches_oracle(ops, oracle, qname):
     assert_matches_f32_reference(actual, exact)
     logical = oracle.grouped(oracle.linear_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n)
     assert nrmse(f32(actual), logical) < FORWARD_TOLERANCE
+    assert max_rel_to_peak(f32(actual), logical) < FORWARD_TOLERANCE
 
 
 @pytest.mark.parametrize("qname", ("Q4_K", "IQ2_S"))
@@ -122,6 +123,9 @@ def test_grouped_forward_group_boundaries(ops, oracle, qname):
     actual = tgo.grouped_mmq(x, device, *_metadata(experts, offsets), qtype, n)
     exact = oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n)
     assert_matches_f32_reference(actual, exact)
+    logical = oracle.grouped(oracle.linear_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n)
+    assert nrmse(f32(actual), logical) < FORWARD_TOLERANCE
+    assert max_rel_to_peak(f32(actual), logical) < FORWARD_TOLERANCE
 
 
 @pytest.mark.parametrize("qname", tuple(QTYPES))

@@ -29,7 +29,12 @@ for entry in (ROOT, ROOT / "torch-ggml-ops_amd"):
 
 import torch  # noqa: E402
 
-PEAK = {"hbm": 8000.0, "int8": 5000.0, "bf16": 2500.0}  # GB/s, TOP/s, TFLOP/s (dense, published)
+PEAK = {"hbm": 8000.0, "int8": 5000.0, "bf16": 2500.0, "fp32_vector": 157.3}  # GB/s, TOP/s, TFLOP/s (dense, published)
+# What the forward algorithm allows: every int8 matrix-core result of a 32-value block needs two fp32 vector
+# operations (x weight-block scale, x activation-block scale + accumulate), and packed fp32 forms are not used,
+# so the vector pipe delivers fp32_vector / 4 lane-operations per second (the published figure counts a fused
+# multiply-add as two and the packed form as two more) and every two of them complete 32 multiply-adds = 64 ops.
+VALU_BOUND_INT8 = PEAK["fp32_vector"] / 4 / 2 * 64  # TOP/s: 1258.4, i.e. 25.2 % of the int8 matrix-core peak
 
 
 def build_pair_workload(device, tokens=8192, experts=256, top_k=8, n=512, k=2048, qtype=13, seed=2024):
@@ -95,30 +100,33 @@ def cpu_baseline_pair(w, budget_seconds=15.0):
     x = w["x"].cpu().float()
     grads = (w["grad_first"].cpu().float(), w["grad_second"].cpu().float())
     weights = (w["first"].cpu().numpy(), w["second"].cpu().numpy())
-    flops, begin, groups = 0.0, 0, 0
+    flops, groups, passes = 0.0, 0, 0
     start = time.perf_counter()
-    for expert, end in zip(indices, offsets):
-        for packed, grad in zip(weights, grads):
-            dense = torch.from_numpy(oracle.dequant_f32(qtype, packed[expert], k))
-            _ = x[begin:end] @ dense.T
-            _ = grad[begin:end] @ dense
-            flops += 2 * 2.0 * (end - begin) * n * k
-        begin = end
-        groups += 1
-        if time.perf_counter() - start > budget_seconds:
-            break
+    while time.perf_counter() - start < budget_seconds:
+        begin = 0
+        for expert, end in zip(indices, offsets):
+            for packed, grad in zip(weights, grads):
+                dense = torch.from_numpy(oracle.dequant_f32(qtype, packed[expert], k))
+                _ = x[begin:end] @ dense.T
+                _ = grad[begin:end] @ dense
+                flops += 2 * 2.0 * (end - begin) * n * k
+            begin = end
+            groups += 1
+            if time.perf_counter() - start > 2 * budget_seconds:
+                break
+        passes += 1
     elapsed = time.perf_counter() - start
     return {
         "value": flops / elapsed / 1e12,
         "unit": "TFLOP/s",
         "cores": threads,
         "kind": "port",
-        "sample": f"first {groups} of {len(indices)} expert groups ({begin} of {w['rows']} rows), "
+        "sample": f"{groups} expert groups in {passes} pass(es) over the workload's {len(indices)} groups ({w['rows']} rows), "
         f"oracle dequant to fp32 + torch.matmul forward and grad-input, {elapsed:.1f} s",
     }
 
 
-def run_decode(args, device) -> None:
+def measure_decode(args, device) -> dict:
     """Decode regime (HBM-bound): T in {1,4,8} tokens x top-8 over 256 experts through the gate+up pair
     (IQ2_S [512,2048]) and the down projection (Q6_K [2048,512]), plus a dense Q3_K [4096,2048] row.
     Every call uses a different seeded routing out of eight, so successive calls touch different experts
@@ -230,6 +238,15 @@ def run_decode(args, device) -> None:
             "gemv_kernel_us": kernel_ms / launches * 1e3,
             "GBps_gemv_kernel": big_bytes / (kernel_ms / launches * 1e-3) / 1e9,
         }
+    for record in report.values():
+        rate = record.get("GBps_gemv_kernels", record.get("GBps_gemv_kernel"))
+        if rate is not None:
+            record["frac_of_hbm_peak"] = rate / PEAK["hbm"]
+    return report
+
+
+def run_decode(args, device) -> None:
+    report = measure_decode(args, device)
     best = max(v.get("GBps_gemv_kernels", v.get("GBps_gemv_kernel", 0.0)) for v in report.values())
     print(json.dumps({
         "metric": "decode-regime weight bandwidth (GEMV kernels), 256-expert MoE shape",
@@ -344,7 +361,7 @@ def run_dense(args, device) -> None:
     }))
 
 
-def run_down(args, device) -> None:
+def measure_down(args, device) -> dict:
     """The down projection of the default workload's model: grouped_mmq, 256 experts, Q4_K [2048, 512],
     4096 tokens x top-8 with the same skewed routing (32 768 rows); forward and grad-input kernel times."""
     import torch_ggml_ops as tgo
@@ -384,6 +401,18 @@ def run_down(args, device) -> None:
         total = sum(times.values())
         result[label] = {"kernels_us": {key: round(value, 1) for key, value in times.items()}, "total_us": round(total, 1),
                          "TFLOPs": round(flops / total / 1e6, 1), "algorithmic_GBps": round(algorithmic / total / 1e3, 1)}
+    result["rows"] = rows
+    result["flops_per_direction"] = flops
+    result["algorithmic_bytes"] = algorithmic
+    # the forward of this shape is HBM-bound on this part (arithmetic intensity 216 FLOP/B, below the ridge)
+    result["forward"]["frac_of_hbm_peak"] = result["forward"]["algorithmic_GBps"] / PEAK["hbm"]
+    result["grad_input"]["frac_of_hbm_peak"] = result["grad_input"]["algorithmic_GBps"] / PEAK["hbm"]
+    return result
+
+
+def run_down(args, device) -> None:
+    result = measure_down(args, device)
+    rows, flops, algorithmic = result.pop("rows"), result.pop("flops_per_direction"), result.pop("algorithmic_bytes")
     both = result["forward"]["total_us"] + result["grad_input"]["total_us"]
     print(json.dumps({
         "metric": "grouped MMQ down projection fwd+bwd throughput (kernel time)", "value": 2 * flops / both / 1e6,
@@ -520,6 +549,8 @@ def main() -> None:
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--no-sub-records", action="store_true",
+                        help="pair workload only: skip the down-projection and decode sub-records")
     parser.add_argument("--workload", choices=("pair", "decode", "multi", "gathered", "layer", "dense", "down"), default="pair")
     parser.add_argument(
         "--quant", choices=("Q3_K", "Q4_K", "Q5_K", "Q6_K", "IQ2_S"), default="Q5_K",
@@ -612,11 +643,16 @@ def main() -> None:
         "frac": achieved / peak,
         "traffic": measured_traffic(dominant) if args.quant == "Q5_K" else None,
         "avg_launch_ms": breakdown[dominant]["avg_ms"],
+        # achieved / what two fp32 vector operations per matrix-core result allow (forward kernel only)
+        "valu_bound": VALU_BOUND_INT8 if dominant == "forward" else None,
+        "valu_bound_frac": achieved / VALU_BOUND_INT8 if dominant == "forward" else None,
     }
     for name in breakdown:
         if name in per_launch:
             b, wk, pk, un = per_launch[name]
             breakdown[name].update({"achieved": wk / (breakdown[name]["avg_ms"] * 1e-3), "unit": un, "frac_of_peak": wk / (breakdown[name]["avg_ms"] * 1e-3) / pk})
+    if "forward" in breakdown:
+        breakdown["forward"]["valu_bound_frac"] = breakdown["forward"]["achieved"] / VALU_BOUND_INT8
 
     result = {
         "metric": "grouped MMQ pair forward+backward throughput, 256-expert MoE shape",
@@ -644,6 +680,21 @@ def main() -> None:
     }
     if not args.no_cpu_baseline:
         result["cpu_baseline"] = cpu_baseline_pair(w)
+    if not args.no_sub_records and args.quant == "Q5_K":
+        # the other configurations of the same model, timed in the same run (kernel time from the event brackets)
+        del w
+        torch.cuda.empty_cache()
+        down = measure_down(args, device)
+        result["down"] = {
+            "workload": f"grouped_mmq down projection: 256 experts, Q4_K [2048,512], T=4096 x top-8 ({down['rows']} rows)",
+            "forward": down["forward"], "grad_input": down["grad_input"],
+        }
+        decode = measure_decode(args, device)
+        result["decode"] = {
+            "workload": "T in {1,4,8} x top-8 over 256 experts: gate+up IQ2_S [512,2048] + down Q6_K [2048,512]; "
+                        "dense Q3_K [4096,2048] M=1; dense Q4_K [28672,8192] M=1..16; weight GB/s of the kernels",
+            "cases": decode,
+        }
     print(json.dumps(result))
 
 

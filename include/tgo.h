@@ -82,6 +82,22 @@ int tgo_mmq_forward(const void * input_bf16, const void * packed, void * output_
                     void * workspace, int64_t rows, int64_t in_features, int64_t out_features,
                     int quant_type, void * stream);
 
+/* tgo_mmq_forward without a workspace argument and without any allocation: the q8_1 activation
+ * workspace is a fixed array inside the library's code object (one copy per GPU, held until the
+ * process ends), TGO_STATIC_WORKSPACE_BYTES large.  Calls whose
+ * tgo_q8_workspace_bytes(rows, in_features) exceeds that are rejected with TGO_ERR_INVALID and a
+ * message; nothing is launched then.  Results are bit-identical to tgo_mmq_forward.  All calls on
+ * one GPU share the array: calls that overlap in time on one GPU (different streams or threads)
+ * race on it and must be serialised by the caller.  The array's address is looked up on the first
+ * call on each device (hipGetSymbolAddress, no allocation), so make that first call outside any
+ * stream capture.  No counterpart in the reference (its dense operator allocates its workspace
+ * through torch, csrc/mmq_hip.cu:646-652); this is for callers that cannot allocate: code under HIP
+ * graph capture, tight serving loops, harnesses that forbid hipMalloc. */
+#define TGO_STATIC_WORKSPACE_BYTES (4 * 1024 * 1024)
+int tgo_mmq_forward_static(const void * input_bf16, const void * packed, void * output_bf16,
+                           int64_t rows, int64_t in_features, int64_t out_features, int quant_type,
+                           void * stream);
+
 /* The second half of tgo_mmq_forward alone: `workspace` already holds the q8_1 form of the
  * activations (written by tgo_quantize_q8_1 for the same rows and in_features) and is only read.
  * Several projections of one input (q/k/v, shared gate/up) quantize once and call this once per

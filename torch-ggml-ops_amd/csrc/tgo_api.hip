@@ -4,6 +4,7 @@
 
 #include <cstdarg>
 #include <cstdio>
+#include <mutex>
 #include <utility>
 #include <vector>
 
@@ -85,6 +86,39 @@ int check_grouped(int64_t num_experts, int64_t num_groups, const void * indices,
     if (indices == nullptr || offsets == nullptr) {
         return fail(TGO_ERR_INVALID, "expert_indices and expert_offsets must not be null");
     }
+    return TGO_OK;
+}
+
+// Activation workspace of tgo_mmq_forward_static: one array per GPU, part of the loaded code object, so the
+// entry point needs no allocation.  In host code the name is only a handle for hipGetSymbolAddress; kernels
+// and copies get the per-device address looked up below.
+constexpr int64_t STATIC_SCRATCH_BYTES = TGO_STATIC_WORKSPACE_BYTES;
+static __device__ __align__(256) uint8_t scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int MAX_DEVICES = 64;
+std::mutex g_scratch_mutex;
+void * g_scratch_address[MAX_DEVICES] = {};
+
+// Address of `scratch` on the current device, looked up once per device (with that device current).
+int static_scratch(void ** address) {
+    int device = -1;
+    const hipError_t status = hipGetDevice(&device);
+    if (status != hipSuccess) {
+        return fail(TGO_ERR_HIP, "hipGetDevice failed: %s", hipGetErrorString(status));
+    }
+    if (device < 0 || device >= MAX_DEVICES) {
+        return fail(TGO_ERR_INVALID, "device ordinal %d is outside the table of static workspaces", device);
+    }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_address[device] == nullptr) {
+        void * found = nullptr;
+        const hipError_t lookup = hipGetSymbolAddress(&found, HIP_SYMBOL(scratch));
+        if (lookup != hipSuccess || found == nullptr) {
+            return fail(TGO_ERR_HIP, "hipGetSymbolAddress(static workspace) failed: %s", hipGetErrorString(lookup));
+        }
+        g_scratch_address[device] = found;
+    }
+    *address = g_scratch_address[device];
     return TGO_OK;
 }
 
@@ -259,6 +293,25 @@ int tgo_mmq_forward(const void * input_bf16, const void * packed, void * output_
                             static_cast<int>(in_features),
                             static_cast<int>(out_features), quant_type, hip_stream),
                      "mmq_forward launch");
+}
+
+int tgo_mmq_forward_static(const void * input_bf16, const void * packed, void * output_bf16, int64_t rows,
+                           int64_t in_features, int64_t out_features, int quant_type, void * stream) {
+    TGO_TRY(check_matmul_shape(rows, in_features, out_features, quant_type));
+    const int64_t needed = tgo::q8_workspace_bytes(rows, in_features);
+    if (needed > STATIC_SCRATCH_BYTES) {
+        return fail(TGO_ERR_INVALID,
+                    "rows x in_features = %lld x %lld needs %lld bytes of activation workspace; the static workspace "
+                    "holds %lld (use tgo_mmq_forward with a caller-provided workspace)",
+                    static_cast<long long>(rows), static_cast<long long>(in_features), static_cast<long long>(needed),
+                    static_cast<long long>(STATIC_SCRATCH_BYTES));
+    }
+    void * workspace = nullptr;
+    TGO_TRY(static_scratch(&workspace));
+    // every byte of the workspace that the multiply kernels read is rewritten by the quantizer of the same
+    // call (padding rows included), so nothing carries over from the previous call
+    return tgo_mmq_forward(input_bf16, packed, output_bf16, workspace, rows, in_features, out_features, quant_type,
+                           stream);
 }
 
 int tgo_mmq_forward_prepared(const void * workspace, const void * packed, void * output_bf16, int64_t rows,

@@ -35,6 +35,7 @@ lib.tgo_dequant_bf16.argtypes = [_p, _p, _i64, _i64, _int, _p]
 lib.tgo_quantize_q8_1.argtypes = [_p, _p, _i64, _i64, _p]
 lib.tgo_q8_workspace_unpack.argtypes = [_p, _p, _p, _p, _i64, _i64, _p]
 lib.tgo_mmq_forward.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _p]
+lib.tgo_mmq_forward_static.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_mmq_forward_prepared.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_grad_workspace_bytes.argtypes = [_i64, _i64, _i64, _int]
 lib.tgo_grad_workspace_bytes.restype = _i64
@@ -67,6 +68,7 @@ EXPORTS = (
     "tgo_quantize_q8_1",
     "tgo_q8_workspace_unpack",
     "tgo_mmq_forward",
+    "tgo_mmq_forward_static",
     "tgo_mmq_forward_prepared",
     "tgo_mmq_grad_input",
     "tgo_grouped_mmq_forward",

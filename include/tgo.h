@@ -54,7 +54,7 @@ int tgo_block_bytes(int quant_type);
 int64_t tgo_q8_workspace_bytes(int64_t rows, int64_t in_features);
 
 /* Bytes of the tile-task list the grouped entry points build on the device
- * (1 counter + 3 int32 per task, at most ceil(rows/tile)+groups tasks, sized for the smallest tile).
+ * (2 counters + 3 int32 per task, at most ceil(rows/tile)+groups tasks, sized for the smallest tile).
  * Replaces new_grouped_row_task_workspace(), csrc/mmq_hip.cu:548-558. */
 int64_t tgo_task_workspace_bytes(int64_t rows, int64_t num_groups);
 

@@ -496,8 +496,10 @@ int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad
     uint8_t * cotangent_first = static_cast<uint8_t *>(workspace) + tgo_task_workspace_bytes(rows, num_groups);
     uint8_t * cotangent_second =
         packed_second != nullptr ? cotangent_first + tgo::cotangent_workspace_bytes(rows, out_features) : nullptr;
+    // tasks of at most BACKWARD_SHORT_ROWS rows go behind the others: a kernel variant of their own runs them
     const tgo::TaskBuild build = {expert_indices, expert_offsets, tasks, static_cast<int>(num_experts),
-                                  static_cast<int>(num_groups), static_cast<int>(rows), row_tile, 0};
+                                  static_cast<int>(num_groups), static_cast<int>(rows), row_tile,
+                                  tgo::BACKWARD_SHORT_ROWS};
     TGO_TRY(check_hip(tgo::launch_pack_cotangent(static_cast<const uint16_t *>(grad_output_first),
                                                  static_cast<const uint16_t *>(grad_output_second), cotangent_first,
                                                  cotangent_second, static_cast<int>(rows),

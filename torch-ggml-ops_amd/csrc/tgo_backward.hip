@@ -28,6 +28,7 @@ namespace tgo {
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 constexpr int BWD_TR = BACKWARD_ROW_TILE;  // rows per workgroup
 constexpr int BWD_TK = 128;                // K columns per workgroup
@@ -111,9 +112,11 @@ struct BackwardArgs {
     int64_t row_bytes;
     uint16_t * dx;
     const int32_t * task_count;   // nullptr: dense
+    const int32_t * task_early;   // tasks listed before the short ones (at most BACKWARD_SHORT_ROWS rows each)
     const int32_t * task_expert;
     const int32_t * task_row_start;
     const int32_t * task_row_end;
+    int segment;        // which tasks of the list a launch runs: 0 all, 1 those before the short ones, 2 the short ones
     int rows;
     int rows_padded;    // rows rounded up to 32: extent of the packed cotangent
     int out_features;   // N, the reduction dimension
@@ -121,6 +124,7 @@ struct BackwardArgs {
     int in_features;    // K
     int k_tiles;        // K / 128
     int task_slots;
+    int short_slots;    // upper bound of the short tasks (one per group at most)
     int sources;        // 1, or 2 for the fused pair
     // Dense calls too small to fill the chip: the reduction over the weight rows is cut into n_splits ranges of
     // steps, blockIdx.y picks one, and the workgroup writes its fp32 sums to partial[split][row][K] instead of
@@ -169,9 +173,29 @@ TGO_DEVICE void decode_k45_octet(const uint8_t * raw, const float2 * scale_min, 
     }
 }
 
-template <int TYPE>
-__global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const BackwardArgs a) {
+// First task and number of tasks of the list's segment that a launch runs.
+TGO_DEVICE void task_segment(const BackwardArgs & a, int & first, int & tasks) {
+    const int count = a.task_count[0];
+    const int early = a.task_early[0];
+    first = a.segment == 2 ? early : 0;
+    tasks = a.segment == 2 ? count - early : a.segment == 1 ? early : count;
+}
+
+// SHORT: the variant for tasks of at most BACKWARD_SHORT_ROWS rows.  Dequantizing a step's weights costs the same
+// however few rows multiply them, so for these tasks it is nearly all of the work: every wave takes the task's 64
+// rows and one 32-column slice of the tile (8 instead of 32 matrix instructions per step, spread over all four
+// SIMDs, 32 accumulator registers instead of 128), and with the smaller register footprint three workgroups share
+// a CU, so that one's barriers and memory waits are covered by another's decoding.
+template <int TYPE, bool SHORT>
+#ifndef TGO_SHORT_OCC
+#define TGO_SHORT_OCC 3
+#endif
+#ifndef TGO_SHORT_DEPTH
+#define TGO_SHORT_DEPTH 1
+#endif
+__global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_grad_input_kernel(const BackwardArgs a) {
     using F = Format<TYPE>;
+    constexpr int KT = SHORT ? 1 : 4;   // 32-column tiles per wave
     constexpr bool FAST_K45 = TYPE == Q4_K || TYPE == Q5_K;
     constexpr int RAW_UNITS = F::BLOCK_BYTES / 16;                              // 16-byte units per block (fast types)
     constexpr int RAW_REGS = (BWD_NS * RAW_UNITS + BWD_THREADS - 1) / BWD_THREADS;  // units in flight per thread
@@ -186,17 +210,22 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
     const int l32 = lane & 31;
     const int half = lane >> 5;
 
-    int k_tile, task;
-    const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + BWD_TR - 1) / BWD_TR;
-    xcd_tile<BWD_XCD_RUN>(blockIdx.x, a.k_tiles, tasks, k_tile, task);
+    int k_tile, task, first_task = 0;
+    int tasks = (a.rows + BWD_TR - 1) / BWD_TR;
+    if (a.task_count != nullptr) {
+        task_segment(a, first_task, tasks);
+    }
+    // (short tasks are remainders of different experts: nothing to gain from runs of tasks per XCD)
+    xcd_tile<SHORT ? 1 : BWD_XCD_RUN>(blockIdx.x, a.k_tiles, tasks, k_tile, task);
     const int kb = k_tile >> 1;          // super-block column
     const int half_block = k_tile & 1;   // which 128 values of it
 
     int expert = 0, row_start, row_end;
     if (a.task_count != nullptr) {
-        if (task >= a.task_count[0]) {
+        if (task >= tasks) {
             return;
         }
+        task += first_task;
         expert = a.task_expert[task];
         row_start = a.task_row_start[task];
         row_end = a.task_row_end[task];
@@ -211,8 +240,9 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
         expand_iq2s_grid(grid, tid, BWD_THREADS);
     }
 
-    const int wave_row = row_start + wave * 64;
-    const bool wave_active = wave_row < row_end;
+    const int wave_row = SHORT ? row_start : row_start + wave * 64;
+    const bool wave_active = SHORT || wave_row < row_end;
+    const int row_tiles = SHORT ? (row_end - row_start + 31) / 32 : 2;   // 32-row tiles this wave multiplies
     const int n_total = a.out_features;
     const int steps_per_source = (n_total + BWD_NS - 1) / BWD_NS;
     const int steps = steps_per_source * a.sources;
@@ -229,24 +259,27 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
         lane_offset[rt] = static_cast<int64_t>(r >> 5) * a.n_chunks * 1024 + ((r & 31) + 32 * half) * 16;
     }
 
-    v16f acc[2][4];
+    v16f acc[2][KT];
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-        for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < KT; ++kt)
 #pragma unroll
             for (int v = 0; v < 16; ++v) acc[rt][kt][v] = 0.0f;
 
     uint4 afrag[2][4] = {};     // cotangent fragments of the step about to be multiplied
-    uint4 raw_regs[FAST_K45 ? RAW_REGS : 1];
+    u32x4 raw_regs[FAST_K45 ? RAW_REGS : 1];   // (a native vector type: arrays of the uint4 struct end up in scratch memory)
 
     // requests the cotangent fragments of a step: chunk s covers columns n0 + 16 s .. + 16
-    auto load_cotangent = [&](int step) {
+    auto load_cotangent = [&](int step) __attribute__((always_inline)) {
         const int source = step / steps_per_source;
         const int n0 = (step - source * steps_per_source) * BWD_NS;
         const uint8_t * base = a.cotangent[source];
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) {
+            if (SHORT && rt >= row_tiles) {
+                break;
+            }
 #pragma unroll
             for (int s = 0; s < 4; ++s) {
                 const int chunk = (n0 >> 4) + s;
@@ -257,7 +290,7 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
         }
     };
     // requests / stores the packed blocks of a step (16-byte aligned types travel through registers)
-    auto load_raw = [&](int step) {
+    auto load_raw = [&](int step) __attribute__((always_inline)) {
         const int source = step / steps_per_source;
         const int n0 = (step - source * steps_per_source) * BWD_NS;
         const uint8_t * weights = a.packed[source] + static_cast<int64_t>(expert) * a.bytes_per_expert;
@@ -270,7 +303,7 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
                 if (row < BWD_NS) {
                     int src_row = n0 + row;
                     src_row = src_row < n_total ? src_row : n_total - 1;
-                    raw_regs[i] = *reinterpret_cast<const uint4 *>(
+                    raw_regs[i] = *reinterpret_cast<const u32x4 *>(
                         weights + src_row * a.row_bytes + static_cast<int64_t>(kb) * F::BLOCK_BYTES + unit * 16);
                 }
             }
@@ -278,7 +311,7 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
             stage_blocks<TYPE>(raw, weights, a.row_bytes, n0, n_total, kb, BWD_NS, tid, BWD_THREADS);
         }
     };
-    auto store_raw = [&]() {
+    auto store_raw = [&]() __attribute__((always_inline)) {
         if constexpr (FAST_K45) {
 #pragma unroll
             for (int i = 0; i < RAW_REGS; ++i) {
@@ -286,13 +319,13 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
                 const int row = id / RAW_UNITS;
                 const int unit = id - row * RAW_UNITS;
                 if (row < BWD_NS) {
-                    *reinterpret_cast<uint4 *>(raw + row * F::RAW_PITCH + unit * 16) = raw_regs[i];
+                    *reinterpret_cast<u32x4 *>(raw + row * F::RAW_PITCH + unit * 16) = raw_regs[i];
                 }
             }
         }
     };
     // dequantizes the staged blocks of a step into one of the two bf16 tiles (ends with the tile visible)
-    auto decode = [&](int step, uint16_t * tile) {
+    auto decode = [&](int step, uint16_t * tile) __attribute__((always_inline)) {
         const int source = step / steps_per_source;
         const int n0 = (step - source * steps_per_source) * BWD_NS;
         __syncthreads();   // staged blocks visible
@@ -334,52 +367,171 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
         __syncthreads();   // tile visible
     };
 
-    // prologue: the first step staged and decoded, its cotangent fragments requested
-    load_raw(step_begin);
-    if (wave_active) {
-        load_cotangent(step_begin);
-    }
-    store_raw();
-    decode(step_begin, wb[0]);
-
-    for (int step = step_begin; step < step_end; ++step) {
-        const bool more = step + 1 < step_end;
-        if (more) {
-            if constexpr (FAST_K45) {
-                load_raw(step + 1);      // in flight during the MFMAs below
+    if constexpr (SHORT && FAST_K45 && TGO_SHORT_DEPTH > 0) {
+        // The multiplications of a step are too short here to cover a memory round trip, so the packed blocks travel
+        // DEPTH steps ahead through a ring of register sets and the cotangent fragments two steps ahead; steps past
+        // the end repeat the last one (harmless re-reads instead of branches around loads).
+        constexpr int DEPTH = TGO_SHORT_DEPTH > 0 ? TGO_SHORT_DEPTH : 1;
+        const int last = step_end - 1;
+        u32x4 ring[DEPTH][RAW_REGS];
+        u32x4 cot[2][2][4] = {};
+        auto request_raw = [&](int step, u32x4 (&regs)[RAW_REGS]) {
+            step = min(step, last);
+            const int source = step / steps_per_source;
+            const int n0 = (step - source * steps_per_source) * BWD_NS;
+            const uint8_t * weights = a.packed[source] + static_cast<int64_t>(expert) * a.bytes_per_expert +
+                                      static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+#pragma unroll
+            for (int i = 0; i < RAW_REGS; ++i) {
+                const int id = min(tid + BWD_THREADS * i, BWD_NS * RAW_UNITS - 1);
+                const int row = id / RAW_UNITS;
+                const int unit = id - row * RAW_UNITS;
+                const int src_row = min(n0 + row, n_total - 1);
+                regs[i] = *reinterpret_cast<const u32x4 *>(weights + src_row * a.row_bytes + unit * 16);
             }
+        };
+        auto park_raw = [&](const u32x4 (&regs)[RAW_REGS]) {
+#pragma unroll
+            for (int i = 0; i < RAW_REGS; ++i) {
+                const int id = tid + BWD_THREADS * i;
+                const int row = id / RAW_UNITS;
+                const int unit = id - row * RAW_UNITS;
+                if (row < BWD_NS) {
+                    *reinterpret_cast<u32x4 *>(raw + row * F::RAW_PITCH + unit * 16) = regs[i];
+                }
+            }
+        };
+        auto request_cotangent = [&](int step, u32x4 (&regs)[2][4]) {
+            step = min(step, last);
+            const int source = step / steps_per_source;
+            const int n0 = (step - source * steps_per_source) * BWD_NS;
+            const uint8_t * base = a.cotangent[source];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt < row_tiles) {
+#pragma unroll
+                    for (int c = 0; c < 4; ++c) {
+                        // (the packed cotangent is zero padded to whole steps of 64 columns)
+                        regs[rt][c] = *reinterpret_cast<const u32x4 *>(
+                            base + lane_offset[rt] + static_cast<int64_t>((n0 >> 4) + c) * 1024);
+                    }
+                }
+            }
+        };
+        auto multiply = [&](const uint16_t * tile, const u32x4 (&regs)[2][4]) {
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const uint4 bits = *reinterpret_cast<const uint4 *>(&tile[(wave * 32 + l32) * BWD_PITCH + 16 * c + 8 * half]);
+                const v8bf bfrag = __builtin_bit_cast(v8bf, bits);
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    if (rt < row_tiles) {
+                        acc[rt][0] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, regs[rt][c]), bfrag,
+                                                                             acc[rt][0], 0, 0, 0);
+                    }
+                }
+            }
+        };
+#pragma unroll
+        for (int d = 0; d < DEPTH; ++d) {
+            request_raw(step_begin + d, ring[d]);
         }
-        if (wave_active) {
-            const uint16_t * tile = wb[(step - step_begin) & 1];
+        request_cotangent(step_begin, cot[0]);
+        request_cotangent(step_begin + 1, cot[1]);
+        park_raw(ring[0]);
+        request_raw(step_begin + DEPTH, ring[0]);
+        decode(step_begin, wb[0]);
+#pragma unroll 1
+        for (int first = step_begin; first < step_end; first += DEPTH) {
 #pragma unroll
-            for (int s = 0; s < 4; ++s) {
-#pragma unroll
-                for (int kt = 0; kt < 4; ++kt) {
-                    const int k = kt * 32 + l32;
-                    const uint4 bits = *reinterpret_cast<const uint4 *>(&tile[k * BWD_PITCH + 16 * s + 8 * half]);
-                    const v8bf bfrag = __builtin_bit_cast(v8bf, bits);
-#pragma unroll
-                    for (int rt = 0; rt < 2; ++rt) {
-                        acc[rt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0);
+            for (int u = 0; u < DEPTH; ++u) {
+                const int step = first + u;
+                if (step < step_end) {
+                    multiply(wb[u & 1], cot[u & 1]);
+                    request_cotangent(step + 2, cot[u & 1]);
+                    if (step + 1 < step_end) {
+                        park_raw(ring[(u + 1) % DEPTH]);
+                        request_raw(step + 1 + DEPTH, ring[(u + 1) % DEPTH]);
+                        decode(step + 1, wb[(u + 1) & 1]);
                     }
                 }
             }
         }
-        if (more) {
-            if (wave_active) {
-                load_cotangent(step + 1);   // in flight while the next tile is decoded
-            }
-            if constexpr (FAST_K45) {
-                store_raw();
-            } else {
-                load_raw(step + 1);
-            }
-            decode(step + 1, wb[(step + 1 - step_begin) & 1]);
+    } else {
+        // prologue: the first step staged and decoded, its cotangent fragments requested
+        load_raw(step_begin);
+        if (wave_active) {
+            load_cotangent(step_begin);
         }
+        store_raw();
+        decode(step_begin, wb[0]);
+
+        for (int step = step_begin; step < step_end; ++step) {
+            const bool more = step + 1 < step_end;
+            if (more) {
+                if constexpr (FAST_K45) {
+                    load_raw(step + 1);      // in flight during the MFMAs below
+                }
+            }
+            if (wave_active) {
+                const uint16_t * tile = wb[(step - step_begin) & 1];
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+#pragma unroll
+                    for (int kt = 0; kt < KT; ++kt) {
+                        const int k = (SHORT ? wave : kt) * 32 + l32;
+                        const uint4 bits = *reinterpret_cast<const uint4 *>(&tile[k * BWD_PITCH + 16 * s + 8 * half]);
+                        const v8bf bfrag = __builtin_bit_cast(v8bf, bits);
+#pragma unroll
+                        for (int rt = 0; rt < 2; ++rt) {
+                            if (SHORT && rt >= row_tiles) {
+                                break;
+                            }
+                            acc[rt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+            if (more) {
+                if (wave_active) {
+                    load_cotangent(step + 1);   // in flight while the next tile is decoded
+                }
+                if constexpr (FAST_K45) {
+                    store_raw();
+                } else {
+                    load_raw(step + 1);
+                }
+                decode(step + 1, wb[(step + 1 - step_begin) & 1]);
+            }
+        }
+
     }
 
     __syncthreads();   // the tiles are free: each wave reuses 8.5 KiB of them to transpose its results
+    if constexpr (SHORT) {
+        // the four 32-column slices of a 32-row tile meet in LDS and leave as whole 256-byte rows
+        constexpr int STAGE_PITCH = BWD_TK + 8;
+        static_assert(2 * 32 * STAGE_PITCH <= 2 * BWD_TK * BWD_PITCH, "both row tiles fit the weight tiles");
+        uint16_t * stage = &wb[0][0];
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            if (rt < row_tiles) {
+                stage_tile_32x32<STAGE_PITCH>(stage + rt * 32 * STAGE_PITCH, acc[rt][0], wave * 32, lane);
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            const int r0 = row_start + rt * 32;
+            if (rt < row_tiles) {
+                store_staged_rows<STAGE_PITCH>(stage + rt * 32 * STAGE_PITCH,
+                                               a.dx + static_cast<int64_t>(r0) * a.in_features + k_tile * BWD_TK,
+                                               a.in_features, row_end - r0, BWD_TK, tid, BWD_THREADS);
+            }
+        }
+        return;
+    } else {
     if (!wave_active) {
         return;
     }
@@ -410,6 +562,7 @@ __global__ __launch_bounds__(BWD_THREADS, 2) void mmq_grad_input_kernel(const Ba
             store_rows_32x128<BWD_TK + 8, true>(stage, acc[rt], a.dx + static_cast<int64_t>(r0) * a.in_features + k_tile * BWD_TK,
                                           a.in_features, row_end - r0, BWD_TK, lane);
         }
+    }
     }
 }
 
@@ -442,7 +595,6 @@ constexpr int BSP_GRID = 256;                      // one workgroup per CU
 // so the prefetches of the role-split kernel are issued and awaited by hand.  Global loads return in order:
 // waiting until at most N of them are outstanding completes everything but the N youngest.  The wait names
 // the awaited registers as read-write operands so that no use of them can be scheduled ahead of it.
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 // `base` must be wave-uniform (it travels in scalar registers); `offset` is this lane's byte offset.
 template <int IMMEDIATE = 0>
@@ -508,8 +660,11 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
         SplitItem item = {0, 0, 0, -1};
         const int64_t linear = blockIdx.x + static_cast<int64_t>(lane) * gridDim.x;
         if (linear < total_items) {
-            int k_tile, task;
-            const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + BWD_TR - 1) / BWD_TR;
+            int k_tile, task, first_task = 0;
+            int tasks = (a.rows + BWD_TR - 1) / BWD_TR;
+            if (a.task_count != nullptr) {
+                task_segment(a, first_task, tasks);   // (never the short segment: first_task is 0)
+            }
             xcd_tile<BWD_XCD_RUN>(static_cast<int>(linear), a.k_tiles, tasks, k_tile, task);
             if (a.task_count != nullptr) {
                 if (task < tasks) {
@@ -911,6 +1066,267 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
     }
 }
 
+// ---- short tasks (Q4_K / Q5_K) --------------------------------------------------------------------------------
+// Tasks of at most BACKWARD_SHORT_ROWS rows.  Dequantizing a step's 64 x 128 weights costs the same however few
+// rows multiply them, so here it is nearly all of the work and every wave does it: a wave owns 16 of the step's 64
+// weight rows from the global load to the bf16 tile (packed blocks DEPTH steps ahead in registers, parked in the
+// wave's own LDS slot, block scales, decode; LDS executes a wave's accesses in order, so these stages need no
+// workgroup barrier), one barrier per step publishes the tile, and then every wave multiplies the task's rows with
+// one 32-column slice of it (4 or 8 matrix instructions).  Small footprint: three workgroups share a CU, so one's
+// barrier and memory waits are covered by the others' decoding.  One workgroup per (task, column tile).
+constexpr int BSH_THREADS = 256;
+constexpr int BSH_ROWS_PER_WAVE = BWD_NS / 4;
+constexpr int BSH_SM_PITCH = BSH_ROWS_PER_WAVE + 1;
+constexpr int BSH_DEPTH = 2;
+
+template <int TYPE>
+__global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(const BackwardArgs a) {
+    using F = Format<TYPE>;
+    static_assert(TYPE == Q4_K || TYPE == Q5_K, "16-byte aligned blocks only");
+    constexpr int RAW_UNITS = F::BLOCK_BYTES / 16;
+    constexpr int RAW_REGS = (BSH_ROWS_PER_WAVE * RAW_UNITS + 63) / 64;
+    constexpr int QS = TYPE == Q4_K ? 16 : 48;
+    __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t raw_all[4][BSH_ROWS_PER_WAVE * F::RAW_PITCH];
+    __shared__ float2 scale_min_all[4][4 * BSH_SM_PITCH];
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+
+    int k_tile, task, first_task, tasks;
+    task_segment(a, first_task, tasks);
+    xcd_tile<1>(blockIdx.x, a.k_tiles, tasks, k_tile, task);
+    if (task >= tasks) {
+        return;
+    }
+    task += first_task;
+    const int expert = a.task_expert[task];
+    const int row_start = a.task_row_start[task];
+    const int row_end = a.task_row_end[task];
+    const int kb = k_tile >> 1;
+    const int half_block = k_tile & 1;
+    const int row_tiles = (row_end - row_start + 31) / 32;   // 1 or 2
+    const int n_total = a.out_features;
+    const int steps_per_source = (n_total + BWD_NS - 1) / BWD_NS;
+    const int steps = steps_per_source * a.sources;
+    const int last = steps - 1;
+
+    uint8_t * const raw = raw_all[wave];
+    float2 * const scale_min = scale_min_all[wave];
+
+    // lane offsets of the 16-byte units this lane fetches per step, relative to the step's first weight row
+    // (the last step of a source clamps rows past the end of the matrix to its last row)
+    const int tail_rows = n_total - (steps_per_source - 1) * BWD_NS;
+    uint32_t unit_offset[RAW_REGS], unit_offset_tail[RAW_REGS];
+#pragma unroll
+    for (int i = 0; i < RAW_REGS; ++i) {
+        const int id = min(lane + 64 * i, BSH_ROWS_PER_WAVE * RAW_UNITS - 1);
+        const int row = wave * BSH_ROWS_PER_WAVE + id / RAW_UNITS;
+        const int unit = id % RAW_UNITS;
+        unit_offset[i] = static_cast<uint32_t>(row * a.row_bytes + unit * 16);
+        unit_offset_tail[i] = static_cast<uint32_t>(min(row, tail_rows - 1) * a.row_bytes + unit * 16);
+    }
+    const int64_t expert_offset = static_cast<int64_t>(expert) * a.bytes_per_expert + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+    auto request = [&](int step, u32x4 (&regs)[RAW_REGS]) __attribute__((always_inline)) {
+        step = min(step, last);
+        const int source = step >= steps_per_source ? 1 : 0;
+        const int n_step = step - source * steps_per_source;
+        const uint8_t * base = (source == 0 ? a.packed[0] : a.packed[1]) + expert_offset +
+                               static_cast<int64_t>(n_step) * BWD_NS * a.row_bytes;
+        const bool tail = n_step == steps_per_source - 1;
+#pragma unroll
+        for (int i = 0; i < RAW_REGS; ++i) {
+            regs[i] = *reinterpret_cast<const u32x4 *>(base + (tail ? unit_offset_tail[i] : unit_offset[i]));
+        }
+    };
+    auto park = [&](const u32x4 (&regs)[RAW_REGS]) __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < RAW_REGS; ++i) {
+            const int id = min(lane + 64 * i, BSH_ROWS_PER_WAVE * RAW_UNITS - 1);
+            const int row = id / RAW_UNITS;
+            const int unit = id - row * RAW_UNITS;
+            uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
+            dst[0] = regs[i].x; dst[1] = regs[i].y; dst[2] = regs[i].z; dst[3] = regs[i].w;
+        }
+    };
+    auto wave_sync = [&]() __attribute__((always_inline)) {
+        __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+    // (d * sc, dmin * m) of this lane's (row, 32-value group); rows past the end of the weight matrix get (0, 0)
+    // and therefore decode to exact zeros
+    auto scales = [&](int step) __attribute__((always_inline)) {
+        const int n = lane & 15;
+        const int group_local = lane >> 4;
+        const uint8_t * blk = raw + n * F::RAW_PITCH;
+        const uint32_t d_dmin = lds_u32(blk), low = lds_u32(blk + 4), mid = lds_u32(blk + 8), high = lds_u32(blk + 12);
+        const int shift = 8 * group_local;
+        const uint32_t b0 = (low >> shift) & 0xffu, b1 = (mid >> shift) & 0xffu, b2 = (high >> shift) & 0xffu;
+        uint32_t sc, mn;
+        if (half_block == 0) {   // groups 0..3 of the super-block: plain 6-bit fields
+            sc = b0 & 63u;
+            mn = b1 & 63u;
+        } else {                 // groups 4..7: low nibbles in the third word, top two bits above the first eight
+            sc = (b2 & 15u) | ((b0 >> 6) << 4);
+            mn = (b2 >> 4) | ((b1 >> 6) << 4);
+        }
+        const int source = step >= steps_per_source ? 1 : 0;
+        const int n0 = (step - source * steps_per_source) * BWD_NS;
+        const bool valid = n0 + wave * BSH_ROWS_PER_WAVE + n < n_total;
+        scale_min[group_local * BSH_SM_PITCH + n] =
+            valid ? make_float2(half_bits_to_float(d_dmin & 0xffffu) * static_cast<float>(sc),
+                                half_bits_to_float(d_dmin >> 16) * static_cast<float>(mn))
+                  : make_float2(0.0f, 0.0f);
+    };
+    // a lane decodes 8 weight rows x 4 consecutive K positions and stores each K position's eight bf16 values with
+    // one 16-byte write
+    const int octet = lane & 1;
+    const int word = (lane >> 1) & 15;
+    const int nibble = lane >> 5;
+    const int position = (word & 7) * 4;
+    const int group_local = 2 * (word >> 3) + nibble;
+    const int group = 4 * half_block + group_local;
+    auto decode = [&](uint16_t * tile) __attribute__((always_inline)) {
+        uint32_t qs[8], qh[8];
+        float2 sm[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int n = 8 * octet + i;
+            const uint8_t * blk = raw + n * F::RAW_PITCH;
+            qs[i] = lds_u32(blk + QS + 64 * half_block + 4 * word);
+            qh[i] = TYPE == Q5_K ? lds_u32(blk + 16 + position) : 0u;
+            sm[i] = scale_min[group_local * BSH_SM_PITCH + n];
+        }
+        float w[4][8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            uint32_t q = (qs[i] >> (4 * nibble)) & 0x0f0f0f0fu;
+            if constexpr (TYPE == Q5_K) {
+                q |= ((qh[i] >> group) & 0x01010101u) << 4;
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                w[e][i] = sm[i].x * static_cast<float>((q >> (8 * e)) & 0xffu) - sm[i].y;
+            }
+        }
+        const int k_local = 32 * group_local + position;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const uint4 packed = make_uint4(pack_bf16x2(w[e][0], w[e][1]), pack_bf16x2(w[e][2], w[e][3]),
+                                            pack_bf16x2(w[e][4], w[e][5]), pack_bf16x2(w[e][6], w[e][7]));
+            *reinterpret_cast<uint4 *>(&tile[(k_local + e) * BWD_PITCH + wave * BSH_ROWS_PER_WAVE + 8 * octet]) = packed;
+        }
+    };
+
+    // cotangent fragments of the task's (up to) two 32-row tiles; one set, requested right after the
+    // multiplications that used the previous one and awaited a whole decode later
+    uint32_t lane_offset[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        int r = row_start + rt * 32 + l32;
+        r = r < a.rows_padded ? r : a.rows_padded - 1;
+        lane_offset[rt] = static_cast<uint32_t>(r >> 5) * a.n_chunks * 1024 + ((r & 31) + 32 * half) * 16;
+    }
+    u32x4 cot[2][4] = {};
+    auto request_cotangent = [&](int step) __attribute__((always_inline)) {
+        step = min(step, last);
+        const int source = step >= steps_per_source ? 1 : 0;
+        const int n0 = (step - source * steps_per_source) * BWD_NS;
+        // (the packed cotangent is zero padded to whole steps of 64 columns)
+        const uint8_t * base = (source == 0 ? a.cotangent[0] : a.cotangent[1]) + static_cast<int64_t>(n0 >> 4) * 1024;
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            if (rt < row_tiles) {
+#pragma unroll
+                for (int c = 0; c < 4; ++c) {
+                    cot[rt][c] = *reinterpret_cast<const u32x4 *>(base + lane_offset[rt] + c * 1024);
+                }
+            }
+        }
+    };
+    v16f acc[2];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[rt][v] = 0.0f;
+    auto multiply = [&](const uint16_t * tile) __attribute__((always_inline)) {
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const uint4 bits = *reinterpret_cast<const uint4 *>(&tile[(wave * 32 + l32) * BWD_PITCH + 16 * c + 8 * half]);
+            const v8bf bfrag = __builtin_bit_cast(v8bf, bits);
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (rt < row_tiles) {
+                    acc[rt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(v8bf, cot[rt][c]), bfrag, acc[rt], 0, 0, 0);
+                }
+            }
+        }
+    };
+
+    u32x4 ring[BSH_DEPTH][RAW_REGS];
+#pragma unroll
+    for (int d = 0; d < BSH_DEPTH; ++d) {
+        request(d, ring[d]);
+    }
+    request_cotangent(0);
+    park(ring[0]);
+    request(BSH_DEPTH, ring[0]);
+    wave_sync();
+    scales(0);
+    wave_sync();
+    decode(wb[0]);
+    __syncthreads();
+#pragma unroll 1
+    for (int first = 0; first < steps; first += BSH_DEPTH) {
+#pragma unroll
+        for (int u = 0; u < BSH_DEPTH; ++u) {
+            const int step = first + u;
+            if (step < steps) {
+                const bool more = step + 1 < steps;
+                if (more) {
+                    // (this wave's decode of the current step, the last reader of its slot, is behind it in program order)
+                    park(ring[(u + 1) % BSH_DEPTH]);
+                    request(step + 1 + BSH_DEPTH, ring[(u + 1) % BSH_DEPTH]);
+                }
+                multiply(wb[u & 1]);
+                request_cotangent(step + 1);
+                if (more) {
+                    wave_sync();
+                    scales(step + 1);
+                    wave_sync();
+                    decode(wb[(u + 1) & 1]);
+                }
+                __syncthreads();
+            }
+        }
+    }
+    // the tiles are free (every wave is past its last multiplication): the four 32-column slices of a 32-row tile
+    // meet in LDS and leave as whole 256-byte rows
+    constexpr int STAGE_PITCH = BWD_TK + 8;
+    static_assert(2 * 32 * STAGE_PITCH <= 2 * BWD_TK * BWD_PITCH, "both row tiles fit the weight tiles");
+    static_assert(BSH_DEPTH % 2 == 0, "tile parity follows the position in the unrolled round");
+    uint16_t * stage = &wb[0][0];
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        if (rt < row_tiles) {
+            stage_tile_32x32<STAGE_PITCH>(stage + rt * 32 * STAGE_PITCH, acc[rt], wave * 32, lane);
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int r0 = row_start + rt * 32;
+        if (rt < row_tiles) {
+            store_staged_rows<STAGE_PITCH>(stage + rt * 32 * STAGE_PITCH,
+                                           a.dx + static_cast<int64_t>(r0) * a.in_features + k_tile * BWD_TK,
+                                           a.in_features, row_end - r0, BWD_TK, tid, BSH_THREADS);
+        }
+    }
+}
+
 // dx[i] = bf16(partial[0][i] + partial[1][i] + ...), eight values per thread; `count` is a multiple of 8.
 __global__ __launch_bounds__(256) void reduce_partials_kernel(const float * __restrict__ partial,
                                                               uint16_t * __restrict__ dx, int64_t count, int n_splits) {
@@ -934,14 +1350,36 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float * __re
 template <int TYPE>
 static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t stream) {
     const int64_t total = static_cast<int64_t>(args.k_tiles) * pad_task_slots(args.task_slots, BWD_XCD_RUN);
-    if (total <= 0 || total > 0x7fffffffLL) {
+    const int64_t total_short = static_cast<int64_t>(args.k_tiles) * pad_task_slots(args.short_slots);
+    if (total <= 0 || total > 0x7fffffffLL || total_short > 0x7fffffffLL) {
         return hipErrorInvalidValue;
     }
     const ProfileScope scope(3, stream);
+    if (args.segment == 1) {
+        // grouped call: the short tasks (a separate segment of the task list) run in a launch of their own
+        BackwardArgs short_args = args;
+        short_args.segment = 2;
+        bool launched = false;
+        if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
+            // (32-bit lane offsets into the packed cotangent and a step's weight rows, as in the role-split kernel)
+            if (cotangent_workspace_bytes(args.rows, args.out_features) < (int64_t{1} << 32) &&
+                args.row_bytes * 2 * BWD_NS < (int64_t{1} << 32)) {
+                mmq_grad_input_short_kernel<TYPE><<<static_cast<unsigned>(total_short), BSH_THREADS, 0, stream>>>(short_args);
+                launched = true;
+            }
+        }
+        if (!launched) {
+            mmq_grad_input_kernel<TYPE, true><<<static_cast<unsigned>(total_short), BWD_THREADS, 0, stream>>>(short_args);
+        }
+        const hipError_t status = hipGetLastError();
+        if (status != hipSuccess) {
+            return status;
+        }
+    }
     if (args.n_splits > 1) {
         // (every format takes the general kernel here: what this path needs is many short workgroups)
         const dim3 grid(static_cast<unsigned>(total), static_cast<unsigned>(args.n_splits));
-        mmq_grad_input_kernel<TYPE><<<grid, BWD_THREADS, 0, stream>>>(args);
+        mmq_grad_input_kernel<TYPE, false><<<grid, BWD_THREADS, 0, stream>>>(args);
         const int64_t count = static_cast<int64_t>(args.rows) * args.in_features;
         reduce_partials_kernel<<<static_cast<unsigned>((count / 8 + 255) / 256), 256, 0, stream>>>(
             args.partial, args.dx, count, args.n_splits);
@@ -961,7 +1399,7 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
             return hipGetLastError();
         }
     }
-    mmq_grad_input_kernel<TYPE><<<static_cast<unsigned>(total), BWD_THREADS, 0, stream>>>(args);
+    mmq_grad_input_kernel<TYPE, false><<<static_cast<unsigned>(total), BWD_THREADS, 0, stream>>>(args);
     return hipGetLastError();
 }
 
@@ -991,12 +1429,19 @@ hipError_t launch_mmq_grad_input(const uint8_t * cotangent_first, const uint8_t 
     args.k_tiles = in_features / BWD_TK;
     if (tasks != nullptr) {
         args.task_count = tasks->count;
+        args.task_early = tasks->early;
         args.task_expert = tasks->expert;
         args.task_row_start = tasks->row_start;
         args.task_row_end = tasks->row_end;
         args.task_slots = tasks->max_tasks;
+        // max_tasks = full row tiles + one remainder per group: the remainders are all that can be short
+        args.short_slots = tasks->max_tasks - (rows + BWD_TR - 1) / BWD_TR;
+        args.segment = 1;
     } else {
         args.task_count = nullptr;
+        args.task_early = nullptr;
+        args.short_slots = 0;
+        args.segment = 0;
         args.task_expert = nullptr;
         args.task_row_start = nullptr;
         args.task_row_end = nullptr;

@@ -11,6 +11,9 @@ namespace tgo {
 // for the single-plane ones.
 static constexpr int forward_row_tile(int quant_type) { return quant_type == 14 || quant_type == 22 ? 256 : 128; }
 constexpr int BACKWARD_ROW_TILE = 256;
+// Grad-input tasks of at most this many rows (a group's remainder) are listed behind the others and run by a
+// kernel variant whose waves split the K columns of the tile instead of its rows.
+constexpr int BACKWARD_SHORT_ROWS = 64;
 // Decode regime: tasks of at most this many rows go to the bandwidth-oriented GEMV kernel.
 constexpr int GEMV_ROW_TILE = 8;
 // Dense calls of up to this many rows take it too, GEMV_ROW_TILE rows at a time: the MFMA kernel's 128-row
@@ -79,9 +82,11 @@ static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t i
     return view;
 }
 
-// Tile tasks of the grouped operators: [count][expert x max][row_start x max][row_end x max].
+// Tile tasks of the grouped operators: [count][early][expert x max][row_start x max][row_end x max].
+// `early` is the number of tasks listed before the short ones (TaskBuild::late_rows); count when nothing is short.
 struct TaskList {
     int32_t * count;
+    int32_t * early;
     int32_t * expert;
     int32_t * row_start;
     int32_t * row_end;
@@ -94,7 +99,7 @@ static inline int max_tasks_for(int64_t rows, int64_t groups, int row_tile) {
 
 static inline int64_t task_workspace_bytes(int64_t rows, int64_t groups) {
     // sized for the smallest tile any kernel uses so one buffer fits every path
-    return (1 + 3 * static_cast<int64_t>(max_tasks_for(rows, groups, GEMV_ROW_TILE))) *
+    return (2 + 3 * static_cast<int64_t>(max_tasks_for(rows, groups, GEMV_ROW_TILE))) *
            static_cast<int64_t>(sizeof(int32_t));
 }
 
@@ -102,7 +107,8 @@ static inline TaskList task_list_view(void * base, int64_t rows, int64_t groups,
     TaskList list;
     list.max_tasks = max_tasks_for(rows, groups, row_tile);
     list.count = static_cast<int32_t *>(base);
-    list.expert = list.count + 1;
+    list.early = list.count + 1;
+    list.expert = list.count + 2;
     list.row_start = list.expert + list.max_tasks;
     list.row_end = list.row_start + list.max_tasks;
     return list;

@@ -117,13 +117,15 @@ int64_t tgo_grad_workspace_bytes(int64_t rows, int64_t out_features, int64_t num
 
 /* Bytes of `workspace` for tgo_mmq_grad_input: the packed cotangent as above, plus, for calls of so
  * few rows that whole reductions per workgroup would leave most of the chip idle, room for the
- * fp32 partial results of a reduction split over several workgroups (added up in a fixed order).
+ * fp32 partial results of a reduction split over several workgroups (added up in a fixed order);
+ * which calls split depends on the format, hence `quant_type`.
  * No counterpart in the reference.  -1 on invalid sizes. */
-int64_t tgo_dense_grad_workspace_bytes(int64_t rows, int64_t out_features, int64_t in_features);
+int64_t tgo_dense_grad_workspace_bytes(int64_t rows, int64_t out_features, int64_t in_features,
+                                       int quant_type);
 
 /* grad_input[rows, in_features] = bf16( grad_output[rows, out_features] x bf16(W) ), weights
  * dequantized to bf16 in LDS, bf16 MFMA, fp32 accumulation, one rounding.
- * `workspace` holds tgo_dense_grad_workspace_bytes(rows, out_features, in_features) bytes.
+ * `workspace` holds tgo_dense_grad_workspace_bytes(rows, out_features, in_features, quant_type) bytes.
  * Replaces launch_dense_mmq_grad_input<type>, csrc/ck/mmq_backward.cuh:1066-1241. */
 int tgo_mmq_grad_input(const void * grad_output_bf16, const void * packed, void * grad_input_bf16,
                        void * workspace, int64_t rows, int64_t out_features, int64_t in_features,

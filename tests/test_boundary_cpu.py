@@ -174,3 +174,19 @@ def test_synthetic_generators_are_seeded_and_well_formed(package, oracle):
     tokens, indices, offsets, weights = synth.zipf_routing(64, 16, 4, seed=5)
     assert tokens.numel() == 256 == int(offsets[-1]) and weights.numel() == 256
     assert (indices[1:] > indices[:-1]).all() and (offsets[1:] > offsets[:-1]).all()
+
+
+def test_token_scatter_masks_rows_outside_the_input(package):
+    """The per-token sum behind the gathered operators' gradients, on the CPU: rows whose index lies outside the
+    token range are dropped (no out-of-range index is ever used), the others add up per token in fp32."""
+    from torch_ggml_ops.gathered import _scatter_to_tokens
+
+    grad_rows = torch.arange(24, dtype=torch.float32).reshape(6, 4).to(torch.bfloat16)
+    row_index = torch.tensor([2, -1, 0, 9, 3, 2])
+    result = _scatter_to_tokens(grad_rows, row_index, 4)
+    expected = torch.zeros(4, 4)
+    for row, token in enumerate(row_index.tolist()):
+        if 0 <= token < 4:
+            expected[token] += grad_rows[row].float()
+    assert result.dtype == torch.bfloat16
+    torch.testing.assert_close(result.float(), expected.to(torch.bfloat16).float(), rtol=0, atol=0)

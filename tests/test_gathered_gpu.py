@@ -111,6 +111,31 @@ def test_gathered_index_outside_the_input_reads_zeros(ops):
     assert torch.count_nonzero(out[1]) == 0 and torch.count_nonzero(out[3]) == 0
 
 
+def test_gathered_gradient_skips_rows_outside_the_input(ops):
+    """Backward through an index with entries outside the token range (dropped tokens): those rows add nothing,
+    the others sum per token as usual, and a second backward returns the same bits."""
+    tgo, synth = ops
+    qtype, n, k = 12, 64, 512
+    weight = synth.random_packed_weight(qtype, (2, n), k, seed=51).cuda()
+    row_index = torch.tensor([2, -1, 0, 9, 3, 2], device="cuda", dtype=torch.int64)
+    indices = torch.tensor([0, 1], device="cuda", dtype=torch.int64)
+    offsets = torch.tensor([2, 6], device="cuda", dtype=torch.int32)
+    grad_output = random_bf16((6, n), seed=53)
+    grads = []
+    for _ in range(2):
+        hidden = random_bf16((4, k), seed=52).requires_grad_(True)
+        tgo.grouped_mmq_gathered(hidden, row_index, weight, indices, offsets, qtype, n).backward(grad_output)
+        grads.append(hidden.grad)
+    torch.testing.assert_close(grads[0], grads[1], rtol=0, atol=0)
+    grad_rows = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default(grad_output, weight, indices, offsets, qtype, k)
+    expected = torch.zeros((4, k), dtype=torch.float64, device="cuda")
+    for row, token in enumerate(row_index.tolist()):
+        if 0 <= token < 4:
+            expected[token] += grad_rows[row].double()
+    torch.testing.assert_close(grads[0].double(), expected, rtol=2**-8, atol=1e-30)
+    assert torch.count_nonzero(grads[0][1]) == 0   # token 1 has no row
+
+
 def test_gathered_rejects_bad_index(ops):
     tgo, synth = ops
     weight = synth.random_packed_weight(12, (2, 32), 256, seed=41).cuda()

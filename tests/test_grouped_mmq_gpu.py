@@ -179,6 +179,53 @@ def test_pair_grad_input_many_tasks_per_workgroup(ops, oracle, qname):
     assert_matches_f32_reference(actual, expected.astype(np.float32), accumulate_noise=2e-6)
 
 
+@pytest.mark.parametrize("sources", (1, 2))
+@pytest.mark.parametrize("n", (64, 128, 192, 200, 296, 512))
+@pytest.mark.parametrize("qname", ("Q4_K", "Q5_K"))
+def test_role_split_kernel_every_prefetch_phase(ops, oracle, qname, n, sources):
+    """The persistent grad-input kernel of Q4_K / Q5_K keeps the packed blocks of four reduction steps and the
+    cotangent fragments of two in flight in rings of registers.  With 1, 2, 3, 4 (200 columns: uneven last step),
+    5 and 8 steps per source, one or two sources and several items per workgroup, every ring phase meets every
+    position in an item; a one-hot cotangent per step must return that step's weight row exactly (bit for bit),
+    and random cotangents must match the oracle.  Groups of 70..300 rows keep the tasks out of the short-task kernel."""
+    tgo, synth = ops
+    qtype, k = QTYPES[qname], 1024
+    sizes = [70, 300, 129]
+    experts, offsets = [2, 0, 3], np.cumsum(sizes).tolist()
+    rows = offsets[-1]
+    host = [synth.random_packed_weight(qtype, (4, n), k, seed=700 + 10 * s + qtype) for s in range(sources)]
+    device = [h.cuda() for h in host]
+    metadata = _metadata(experts, offsets)
+    op_single = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default
+    op_pair = torch.ops.torch_ggml_ops.grouped_mmq_pair_grad_input.default
+
+    def run(grads):
+        if sources == 1:
+            return op_single(grads[0], device[0], *metadata, qtype, k)
+        return op_pair(grads[0], grads[1], device[0], device[1], *metadata, qtype, k)
+
+    logical = [oracle.bf16_to_f32(oracle.dequant_bf16(qtype, h.numpy(), k)) for h in host]   # [experts, n, k]
+    steps = (n + 63) // 64
+    # row r of group g gets a one in column (64 * (r % steps) + r % 64) capped at n - 1 of source r % sources
+    one_hot = [torch.zeros(rows, n, dtype=torch.bfloat16) for _ in range(sources)]
+    picks, begin = [], 0
+    for expert, end in zip(experts, offsets):
+        for row in range(begin, end):
+            column = min(64 * (row % steps) + row % 64, n - 1)
+            one_hot[row % sources][row, column] = 1
+            picks.append((row, expert, row % sources, column))
+        begin = end
+    result = f32(run([g.cuda() for g in one_hot]))
+    for row, expert, source, column in picks:
+        np.testing.assert_array_equal(result[row], logical[source][expert, column], err_msg=f"row {row} column {column}")
+
+    grads = [random_bf16((rows, n), seed=900 + s) for s in range(sources)]
+    expected = np.zeros((rows, k), dtype=np.float64)
+    for s in range(sources):
+        expected += oracle.grouped(oracle.grad_input, qtype, bits(grads[s]), host[s].numpy(), experts, offsets, n, k, k)
+    assert_matches_f32_reference(run(grads), expected.astype(np.float32), accumulate_noise=2e-6)
+
+
 @pytest.mark.parametrize("qname", ("Q4_K", "Q6_K"))
 def test_more_groups_than_one_listing_pass(ops, oracle, qname):
     """700 groups: the tile-task list is written 256 groups at a time, and the forward lists tasks of at most

@@ -122,7 +122,11 @@ int static_scratch(void ** address) {
     return TGO_OK;
 }
 
+// Opt-in launch timing.  The lists are shared by every thread that launches; the mutex guards them, and a list
+// stops growing at PROFILE_EVENT_LIMIT brackets (later launches go untimed until the next tgo_profile_enable).
 bool g_profile = false;
+std::mutex g_profile_mutex;
+constexpr size_t PROFILE_EVENT_LIMIT = 1 << 16;
 std::vector<std::pair<hipEvent_t, hipEvent_t>> g_profile_events[TGO_KERNEL_COUNT];
 
 void drop_profile_events() {
@@ -149,7 +153,16 @@ namespace tgo {
 
 ProfileScope::ProfileScope(int kernel_id, hipStream_t launch_stream)
     : kernel(kernel_id), stream(launch_stream), start(nullptr), active(false) {
-    if (g_profile && hipEventCreate(&start) == hipSuccess) {
+    if (!g_profile) {
+        return;
+    }
+    {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
+        if (g_profile_events[kernel].size() >= PROFILE_EVENT_LIMIT) {
+            return;
+        }
+    }
+    if (hipEventCreate(&start) == hipSuccess) {
         active = hipEventRecord(start, stream) == hipSuccess;
         if (!active) {
             (void)hipEventDestroy(start);
@@ -163,6 +176,7 @@ ProfileScope::~ProfileScope() {
     }
     hipEvent_t stop = nullptr;
     if (hipEventCreate(&stop) == hipSuccess && hipEventRecord(stop, stream) == hipSuccess) {
+        std::lock_guard<std::mutex> lock(g_profile_mutex);
         g_profile_events[kernel].emplace_back(start, stop);
     } else {
         (void)hipEventDestroy(start);
@@ -179,6 +193,7 @@ extern "C" {
 int tgo_version(void) { return 100; }
 
 int tgo_profile_enable(int enabled) {
+    std::lock_guard<std::mutex> lock(g_profile_mutex);
     drop_profile_events();
     g_profile = enabled != 0;
     return TGO_OK;
@@ -189,6 +204,7 @@ int tgo_profile_read(int kernel, double * total_ms, int64_t * launches) {
         return fail(TGO_ERR_INVALID, "bad profile query");
     }
     double total = 0.0;
+    std::lock_guard<std::mutex> lock(g_profile_mutex);
     for (auto & pair : g_profile_events[kernel]) {
         TGO_TRY(check_hip(hipEventSynchronize(pair.second), "hipEventSynchronize"));
         float ms = 0.0f;
@@ -219,12 +235,13 @@ int64_t tgo_task_workspace_bytes(int64_t rows, int64_t num_groups) {
     return (tgo::task_workspace_bytes(rows, num_groups) + 15) / 16 * 16;
 }
 
-int64_t tgo_dense_grad_workspace_bytes(int64_t rows, int64_t out_features, int64_t in_features) {
-    if (rows <= 0 || out_features <= 0 || in_features <= 0 || in_features % tgo::QK_K != 0) {
+int64_t tgo_dense_grad_workspace_bytes(int64_t rows, int64_t out_features, int64_t in_features, int quant_type) {
+    if (rows <= 0 || out_features <= 0 || in_features <= 0 || in_features % tgo::QK_K != 0 ||
+        tgo::block_bytes(quant_type) == 0) {
         return -1;
     }
     return (tgo::cotangent_workspace_bytes(rows, out_features) + 15) / 16 * 16 +
-           tgo::dense_grad_partial_bytes(rows, out_features, in_features);
+           tgo::dense_grad_partial_bytes(rows, out_features, in_features, quant_type);
 }
 
 int64_t tgo_grad_workspace_bytes(int64_t rows, int64_t out_features, int64_t num_groups, int sources) {
@@ -345,8 +362,9 @@ int tgo_mmq_grad_input(const void * grad_output_bf16, const void * packed, void 
                                                  hip_stream),
                       "pack_cotangent launch"));
     // scratch for the split reduction of small calls follows the packed cotangent
-    float * partial = reinterpret_cast<float *>(
-        cotangent + (tgo::cotangent_workspace_bytes(rows, out_features) + 15) / 16 * 16);
+    float * partial = tgo::dense_grad_partial_bytes(rows, out_features, in_features, quant_type) > 0
+        ? reinterpret_cast<float *>(cotangent + (tgo::cotangent_workspace_bytes(rows, out_features) + 15) / 16 * 16)
+        : nullptr;
     return check_hip(tgo::launch_mmq_grad_input(cotangent, nullptr, static_cast<const uint8_t *>(packed), nullptr, 0,
                                                 static_cast<uint16_t *>(grad_input_bf16), nullptr,
                                                 static_cast<int>(rows), static_cast<int>(out_features),

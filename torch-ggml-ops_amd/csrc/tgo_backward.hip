@@ -1412,7 +1412,7 @@ hipError_t launch_mmq_grad_input(const uint8_t * cotangent_first, const uint8_t 
     // `partial` (dense calls only): room for dense_grad_splits() fp32 copies of the result, or nullptr
     args.partial = partial;
     args.n_splits = tasks == nullptr && partial != nullptr
-        ? dense_grad_splits(rows, out_features, in_features, quant_type == Q4_K || quant_type == Q5_K) : 1;
+        ? dense_grad_splits(rows, out_features, in_features, has_role_split(quant_type)) : 1;
     args.cotangent[0] = cotangent_first;
     args.cotangent[1] = cotangent_second;
     args.packed[0] = packed_first;

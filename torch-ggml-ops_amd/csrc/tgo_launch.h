@@ -39,9 +39,11 @@ static inline int dense_grad_splits(int64_t rows, int64_t out_features, int64_t 
     splits = splits < 16 ? splits : 16;
     return splits < 2 ? 1 : static_cast<int>(splits);
 }
-// (sized for the formats that split most)
-static inline int64_t dense_grad_partial_bytes(int64_t rows, int64_t out_features, int64_t in_features) {
-    const int splits = dense_grad_splits(rows, out_features, in_features, false);
+// Q4_K (12) and Q5_K (13) have the role-split kernel.
+static inline bool has_role_split(int quant_type) { return quant_type == 12 || quant_type == 13; }
+// fp32 scratch of the split reduction for a dense call of this format: the same decision as the launcher's
+static inline int64_t dense_grad_partial_bytes(int64_t rows, int64_t out_features, int64_t in_features, int quant_type) {
+    const int splits = dense_grad_splits(rows, out_features, in_features, has_role_split(quant_type));
     return splits > 1 ? splits * rows * in_features * 4 : 0;
 }
 

@@ -39,7 +39,7 @@ lib.tgo_mmq_forward_static.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_mmq_forward_prepared.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_grad_workspace_bytes.argtypes = [_i64, _i64, _i64, _int]
 lib.tgo_grad_workspace_bytes.restype = _i64
-lib.tgo_dense_grad_workspace_bytes.argtypes = [_i64, _i64, _i64]
+lib.tgo_dense_grad_workspace_bytes.argtypes = [_i64, _i64, _i64, _int]
 lib.tgo_dense_grad_workspace_bytes.restype = _i64
 lib.tgo_mmq_grad_input.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_grouped_mmq_forward.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]

@@ -8,8 +8,9 @@ quantizer reads row ``row_index[r]`` of the token activations directly, so the s
 exists; results are bit-identical to ``grouped_mmq(hidden.index_select(0, row_index), ...)``.
 
 The gradient with respect to the token activations is the grouped grad-input of the sorted rows
-summed back per token in fp32 and rounded once.  ``row_index`` must hold valid token rows, as for
-``index_select``.
+summed back per token in fp32 and rounded once.  An entry of ``row_index`` outside ``[0, tokens)``
+(for example -1 for a dropped token) reads as a row of zeros in the forward and receives no
+gradient in the backward.
 """
 
 from __future__ import annotations
@@ -70,9 +71,18 @@ def _rows_grad_input(first_grad, second_grad, first_weight, second_weight, exper
 
 
 def _scatter_to_tokens(grad_rows: torch.Tensor, row_index: torch.Tensor, tokens: int) -> torch.Tensor:
-    """Sum of the sorted rows' gradients per token: fp32 accumulation, one rounding to bf16."""
+    """Sum of the sorted rows' gradients per token: fp32 accumulation, one rounding to bf16.
+
+    Rows whose index lies outside ``[0, tokens)`` were zeros in the forward and are dropped here (the index
+    is clamped and the row masked, so no out-of-range index reaches the device).  The sum runs through
+    ``index_put_(accumulate=True)``, which sorts the indices and adds each token's rows in row order: the
+    result does not depend on scheduling, unlike the atomic adds of ``index_add_``.
+    """
+    present = (row_index >= 0) & (row_index < tokens)
+    safe = row_index.clamp(0, tokens - 1)
+    values = grad_rows.float() * present.unsqueeze(1)
     total = torch.zeros((tokens, grad_rows.shape[1]), dtype=torch.float32, device=grad_rows.device)
-    total.index_add_(0, row_index, grad_rows.float())
+    total.index_put_((safe,), values, accumulate=True)
     return total.to(grad_rows.dtype)
 
 

@@ -51,7 +51,7 @@ def _mmq_grad_input_device(
     with torch.cuda.device(grad_output.device):
         grad_input = grad_output.new_empty((*grad_output.shape[:-1], in_features))
         workspace = grad_output.new_empty(
-            (_native.lib.tgo_dense_grad_workspace_bytes(rows, out_features, in_features),), dtype=torch.uint8
+            (_native.lib.tgo_dense_grad_workspace_bytes(rows, out_features, in_features, quant_type),), dtype=torch.uint8
         )
         _native.check(
             _native.lib.tgo_mmq_grad_input(

@@ -5,7 +5,8 @@ six ``torch_ggml_ops::`` operators of the reference with their fake kernels and 
 plus ``quantize_q8_1`` / ``mmq_prepared`` for several projections of one input and the
 ``*_gathered`` grouped operators that fold the token -> sorted-row gather into the quantizer,
 the routing sort / weighted combine of a mixture-of-experts layer (``route``, ``moe_combine``, ``moe_layer``)
-and ``grouped_mmq_swiglu``, the gate/up pair with the activation fused into the kernel's epilogue.
+``grouped_mmq_swiglu``, the gate/up pair with the activation fused into the kernel's epilogue, and
+``chunked_lm_head_loss``, the cross-entropy through a packed LM head one chunk of rows at a time.
 """
 
 import torch  # noqa: F401  (operators are registered against the loaded torch)
@@ -13,12 +14,14 @@ import torch  # noqa: F401  (operators are registered against the loaded torch)
 from . import _native  # noqa: F401  loads libtgo_hip.so or fails loudly
 from .gathered import grouped_mmq_gathered, grouped_mmq_pair_gathered
 from .grouped_mmq import grouped_mmq, grouped_mmq_pair
+from .lm_head import chunked_lm_head_loss
 from .mmq import mmq
 from .moe import moe_combine, moe_layer, route
 from .prepared import mmq_multi, mmq_prepared, quantize_q8_1
 from .swiglu import grouped_mmq_swiglu
 
 __all__ = [
+    "chunked_lm_head_loss",
     "grouped_mmq",
     "grouped_mmq_gathered",
     "grouped_mmq_pair",

@@ -526,6 +526,29 @@ def run_layer(args, device) -> None:
         if launches:
             kernels[name] = {"avg_ms": total_ms / launches, "launches_per_step": launches / args.steps}
     _native.lib.tgo_profile_enable(0)
+    # forward + backward of the layer (gradient of the token activations), with the down projection and the
+    # combine as one step (its backward gathers and scales the per-token gradient while packing the cotangent)
+    # against the two separate operators (whose backward builds the expert-sorted gradient with torch operators)
+    grad_out = torch.randn(tokens, features, device=device, generator=generator).to(torch.bfloat16)
+
+    def two_step_layer(x):
+        row_index, slot_rows, expert_indices, expert_offsets = tgo.route(slot_experts, experts)
+        activated = tgo.grouped_mmq_swiglu(x, gate, up, expert_indices, expert_offsets, qtype, intermediate, row_index)
+        rows_out = tgo.grouped_mmq(activated, down, expert_indices, expert_offsets, qtype, features)
+        return tgo.moe_combine(rows_out, slot_rows, slot_weights)
+
+    training = {}
+    for name, fn in (("fused_down_combine", lambda x: tgo.moe_layer(x, slot_experts, slot_weights, gate, up, down, qtype, qtype, intermediate)),
+                     ("two_step_combine", two_step_layer)):
+        x = hidden.clone().requires_grad_(True)
+        for _ in range(args.warmup):
+            fn(x).backward(grad_out)
+        torch.cuda.synchronize()
+        start = time.perf_counter()
+        for _ in range(args.steps):
+            fn(x).backward(grad_out)
+        torch.cuda.synchronize()
+        training[name + "_fwd_bwd_ms"] = (time.perf_counter() - start) / args.steps * 1e3
     rows = tokens * top_k
     combine_bytes = 2.0 * features * (rows + tokens) + 12.0 * rows
     combine_rate = combine_bytes / (kernels["combine"]["avg_ms"] * 1e-3) / 1e9
@@ -540,6 +563,7 @@ def run_layer(args, device) -> None:
                                f"T=8192 x top-8 ({rows} sorted rows)"},
         "kernels": kernels,
         "caller_side_activation_ms": unfused * 1e3,
+        "training": training,
     }))
 
 

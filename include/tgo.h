@@ -199,6 +199,22 @@ int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad
                                int64_t out_features, int64_t in_features, int64_t num_experts,
                                int64_t num_groups, int quant_type, void * stream);
 
+/* tgo_grouped_mmq_grad_input (single projection) with the routing-weighted return of a mixture-of-experts
+ * layer, run backwards, folded into the cotangent's packing: cotangent row r of the operator is
+ *   bf16( row_weight[r] * grad_tokens[row_token[r], :] )        (fp32 product, one rounding)
+ * with grad_tokens bf16 [tokens, out_features] the gradient of the layer's per-token output, row_token int64
+ * [rows] the token of each expert-sorted row and row_weight fp32 [rows] its routing weight; a row whose token
+ * lies outside [0, tokens) has a zero cotangent.  The expert-sorted cotangent that the caller would otherwise
+ * build from the gradient of tgo_moe_combine (rows x out_features bf16, written and read again) is never
+ * materialised.  Same workspace as tgo_grouped_mmq_grad_input with one source.  No counterpart in the reference,
+ * which leaves the combine and its gradient to the caller (torch_ggml_ops/grouped_mmq.py:216). */
+int tgo_grouped_mmq_grad_input_weighted(const void * grad_tokens_bf16, const int64_t * row_token,
+                                        const float * row_weight, int64_t tokens, const void * packed,
+                                        void * grad_input_bf16, const int64_t * expert_indices,
+                                        const int32_t * expert_offsets, void * workspace, int64_t rows,
+                                        int64_t out_features, int64_t in_features, int64_t num_experts,
+                                        int64_t num_groups, int quant_type, void * stream);
+
 /* Name of the kernel family the forward entry points pick for a shape ("mfma" or "gemv");
  * host pointer to a static string.  Lets callers and benchmarks label what they measure. */
 const char * tgo_forward_kernel_family(int64_t rows, int64_t num_groups);

@@ -138,3 +138,70 @@ def test_layer_matches_float64_on_dequantized_weights(ops, oracle, gate_up, down
     out.backward(grad)
     expected.backward(grad.double().cpu())
     assert nrmse(f32(hidden.grad), x.grad.float().numpy()) < 2e-2
+
+
+@pytest.mark.parametrize("qname", ("Q4_K", "Q6_K"))
+def test_projection_with_combine_equals_the_two_steps(ops, oracle, qname):
+    """grouped_mmq_combine = moe_combine(grouped_mmq(...)): same bits forward, and a backward whose cotangent
+    packing gathers the per-token gradient and applies the routing weight itself.  Checked against the two
+    separate operators bit for bit, and against a float64 restatement on oracle-dequantized weights."""
+    tgo, synth = ops
+    qtype, tokens, top_k, experts, k, n = QTYPES[qname], 150, 3, 7, 512, 200
+    host = synth.random_packed_weight(qtype, (experts, n), k, seed=71)
+    weight = host.cuda()
+    slot_experts, slot_weights = _choices(tokens, top_k, experts, seed=72)
+    _row_index, slot_rows, indices, offsets = tgo.route(slot_experts, experts)
+    rows = tokens * top_k
+    grad = random_bf16((tokens, n), seed=74)
+
+    fused_in = random_bf16((rows, k), seed=73).requires_grad_(True)
+    fused_w = slot_weights.clone().requires_grad_(True)
+    fused = tgo.grouped_mmq_combine(fused_in, weight, indices, offsets, slot_rows, fused_w, qtype, n)
+    fused.backward(grad)
+
+    plain_in = random_bf16((rows, k), seed=73).requires_grad_(True)
+    plain_w = slot_weights.clone().requires_grad_(True)
+    plain = tgo.moe_combine(tgo.grouped_mmq(plain_in, weight, indices, offsets, qtype, n), slot_rows, plain_w)
+    plain.backward(grad)
+
+    torch.testing.assert_close(fused, plain, rtol=0, atol=0)
+    torch.testing.assert_close(fused_in.grad, plain_in.grad, rtol=0, atol=0)
+    torch.testing.assert_close(fused_w.grad, plain_w.grad, rtol=0, atol=0)
+
+    # d/d(input row r) = w[r] * grad[token of r] @ bf16(W[expert of r]), the cotangent rounded to bf16 first
+    dense = np.stack([oracle.bf16_to_f32(oracle.dequant_bf16(qtype, host[e].numpy(), k)) for e in range(experts)]).astype(np.float64)
+    slot_of_row = np.empty(rows, dtype=np.int64)
+    slot_of_row[slot_rows.reshape(-1).cpu().numpy()] = np.arange(rows)
+    grad64, weights64 = grad.double().cpu().numpy(), slot_weights.double().cpu().numpy().reshape(-1)
+    expert_of_slot = slot_experts.reshape(-1).cpu().numpy()
+    expected = np.empty((rows, k))
+    for r in range(rows):
+        slot = slot_of_row[r]
+        cotangent = (torch.from_numpy(weights64[slot] * grad64[slot // top_k]).float().bfloat16().double().numpy())
+        expected[r] = cotangent @ dense[expert_of_slot[slot]]
+    assert_matches_f32_reference(fused_in.grad, expected.astype(np.float32), accumulate_noise=2e-6)
+
+
+def test_weighted_grad_input_skips_rows_without_a_token(ops):
+    tgo, synth = ops
+    qtype, k, n = 12, 256, 64
+    weight = synth.random_packed_weight(qtype, (2, n), k, seed=75).cuda()
+    grad_tokens = random_bf16((3, n), seed=76)
+    row_token = torch.tensor([2, -1, 0, 5, 1], device="cuda", dtype=torch.int64)
+    row_weight = torch.tensor([0.5, 3.0, 2.0, 7.0, 1.0], device="cuda")
+    indices = torch.tensor([1, 0], device="cuda", dtype=torch.int64)
+    offsets = torch.tensor([2, 5], device="cuda", dtype=torch.int32)
+    actual = torch.ops.torch_ggml_ops.grouped_mmq_grad_input_weighted.default(
+        grad_tokens, row_token, row_weight, weight, indices, offsets, qtype, k
+    )
+    sorted_grad = torch.zeros((5, n), device="cuda", dtype=torch.bfloat16)
+    for row, (token, factor) in enumerate(zip(row_token.tolist(), row_weight.tolist())):
+        if 0 <= token < 3:
+            sorted_grad[row] = (grad_tokens[token].float() * factor).bfloat16()
+    expected = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default(sorted_grad, weight, indices, offsets, qtype, k)
+    torch.testing.assert_close(actual, expected, rtol=0, atol=0)
+    assert torch.count_nonzero(actual[1]) == 0 and torch.count_nonzero(actual[3]) == 0
+    with pytest.raises(RuntimeError, match="row_weight"):
+        torch.ops.torch_ggml_ops.grouped_mmq_grad_input_weighted.default(
+            grad_tokens, row_token, row_weight.double(), weight, indices, offsets, qtype, k
+        )

@@ -487,11 +487,13 @@ int tgo_moe_combine(const void * rows_bf16, const int64_t * slot_rows, const flo
                      "moe_combine launch");
 }
 
-int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad_output_second,
-                               const void * packed_first, const void * packed_second, void * grad_input_bf16,
-                               const int64_t * expert_indices, const int32_t * expert_offsets,
-                               void * workspace, int64_t rows, int64_t out_features, int64_t in_features,
-                               int64_t num_experts, int64_t num_groups, int quant_type, void * stream) {
+// Shared body of the grouped grad-input entry points; `row_token` is null for a cotangent given row by row.
+static int grouped_grad_input(const void * grad_output_first, const void * grad_output_second,
+                              const int64_t * row_token, const float * row_weight, int64_t tokens,
+                              const void * packed_first, const void * packed_second, void * grad_input_bf16,
+                              const int64_t * expert_indices, const int32_t * expert_offsets, void * workspace,
+                              int64_t rows, int64_t out_features, int64_t in_features, int64_t num_experts,
+                              int64_t num_groups, int quant_type, void * stream) {
     TGO_TRY(check_matmul_shape(rows, in_features, out_features, quant_type));
     TGO_TRY(check_grouped(num_experts, num_groups, expert_indices, expert_offsets));
     TGO_TRY(check_pointer(grad_output_first, "grad_output"));
@@ -521,7 +523,8 @@ int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad
     TGO_TRY(check_hip(tgo::launch_pack_cotangent(static_cast<const uint16_t *>(grad_output_first),
                                                  static_cast<const uint16_t *>(grad_output_second), cotangent_first,
                                                  cotangent_second, static_cast<int>(rows),
-                                                 static_cast<int>(out_features), hip_stream, &build),
+                                                 static_cast<int>(out_features), hip_stream, &build, row_token,
+                                                 row_weight, tokens),
                       "pack_cotangent launch"));
     return check_hip(tgo::launch_mmq_grad_input(cotangent_first, cotangent_second,
                                                 static_cast<const uint8_t *>(packed_first),
@@ -530,6 +533,33 @@ int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad
                                                 static_cast<int>(rows), static_cast<int>(out_features),
                                                 static_cast<int>(in_features), quant_type, hip_stream),
                      "grouped mmq_grad_input launch");
+}
+
+int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad_output_second,
+                               const void * packed_first, const void * packed_second, void * grad_input_bf16,
+                               const int64_t * expert_indices, const int32_t * expert_offsets,
+                               void * workspace, int64_t rows, int64_t out_features, int64_t in_features,
+                               int64_t num_experts, int64_t num_groups, int quant_type, void * stream) {
+    return grouped_grad_input(grad_output_first, grad_output_second, nullptr, nullptr, 0, packed_first, packed_second,
+                              grad_input_bf16, expert_indices, expert_offsets, workspace, rows, out_features,
+                              in_features, num_experts, num_groups, quant_type, stream);
+}
+
+int tgo_grouped_mmq_grad_input_weighted(const void * grad_tokens_bf16, const int64_t * row_token,
+                                        const float * row_weight, int64_t tokens, const void * packed,
+                                        void * grad_input_bf16, const int64_t * expert_indices,
+                                        const int32_t * expert_offsets, void * workspace, int64_t rows,
+                                        int64_t out_features, int64_t in_features, int64_t num_experts,
+                                        int64_t num_groups, int quant_type, void * stream) {
+    if (row_token == nullptr || row_weight == nullptr) {
+        return fail(TGO_ERR_INVALID, "row_token and row_weight must not be null");
+    }
+    if (tokens <= 0) {
+        return fail(TGO_ERR_INVALID, "tokens must be positive; got %lld", static_cast<long long>(tokens));
+    }
+    return grouped_grad_input(grad_tokens_bf16, nullptr, row_token, row_weight, tokens, packed, nullptr,
+                              grad_input_bf16, expert_indices, expert_offsets, workspace, rows, out_features,
+                              in_features, num_experts, num_groups, quant_type, stream);
 }
 
 }  // extern "C"

@@ -41,11 +41,21 @@ static_assert(BWD_TR == 64 * BWD_THREADS / 64, "64 rows per wave");
 // ---- cotangent packing ---------------------------------------------------------------------------------
 // One workgroup handles 32 rows x 128 columns (8 slabs): coalesced row reads, transpose through LDS,
 // one contiguous 8 KiB write.
+// With `gather` set (single cotangent only), row r of the cotangent is bf16(scale[r] * grad_first[gather[r], :]):
+// the routing-weighted return of a mixture-of-experts layer run backwards, read straight from the per-token
+// cotangent (rows whose index lies outside [0, gather_rows) are zeros), so the expert-sorted cotangent that the
+// caller would otherwise build (rows x out_features bf16 written and read again) never exists.
+TGO_DEVICE uint32_t scale_bf16x2(uint32_t pair, float scale) {
+    return pack_bf16x2(scale * bf16_bits_to_float(pair & 0xffffu), scale * bf16_bits_to_float(pair >> 16));
+}
+
 __global__ __launch_bounds__(256) void pack_cotangent_kernel(const uint16_t * __restrict__ grad_first,
                                                             const uint16_t * __restrict__ grad_second,
                                                             uint8_t * __restrict__ packed_first,
                                                             uint8_t * __restrict__ packed_second, int rows,
-                                                            int out_features, int n_chunks, const TaskBuild build) {
+                                                            int out_features, int n_chunks, const TaskBuild build,
+                                                            const int64_t * __restrict__ gather,
+                                                            const float * __restrict__ scale, int64_t gather_rows) {
     __shared__ __attribute__((aligned(16))) uint8_t tile[8 * 1024];
     if (build.tasks.count != nullptr && blockIdx.x == 0 && blockIdx.y == 0 && blockIdx.z == 0) {
         build_tasks(build, threadIdx.x);
@@ -60,8 +70,16 @@ __global__ __launch_bounds__(256) void pack_cotangent_kernel(const uint16_t * __
     const int row = row_tile * 32 + rr;
     const int n = (chunk0 + c) * 16;
     uint4 lo = make_uint4(0, 0, 0, 0), hi = make_uint4(0, 0, 0, 0);
-    if (row < rows && n < out_features) {
-        const uint16_t * src = grad + static_cast<int64_t>(row) * out_features + n;
+    int64_t source_row = row;
+    float factor = 1.0f;
+    bool present = row < rows && n < out_features;
+    if (gather != nullptr && present) {   // (uniform: one launch either gathers or does not)
+        source_row = gather[row];
+        factor = scale[row];
+        present = source_row >= 0 && source_row < gather_rows;
+    }
+    if (present) {
+        const uint16_t * src = grad + source_row * out_features + n;
         if ((out_features & 7) == 0 && n + 16 <= out_features) {
             lo = *reinterpret_cast<const uint4 *>(src);
             hi = *reinterpret_cast<const uint4 *>(src + 8);
@@ -73,6 +91,10 @@ __global__ __launch_bounds__(256) void pack_cotangent_kernel(const uint16_t * __
             }
             lo = make_uint4(e[0] | (e[1] << 16), e[2] | (e[3] << 16), e[4] | (e[5] << 16), e[6] | (e[7] << 16));
             hi = make_uint4(e[8] | (e[9] << 16), e[10] | (e[11] << 16), e[12] | (e[13] << 16), e[14] | (e[15] << 16));
+        }
+        if (gather != nullptr) {
+            lo = make_uint4(scale_bf16x2(lo.x, factor), scale_bf16x2(lo.y, factor), scale_bf16x2(lo.z, factor), scale_bf16x2(lo.w, factor));
+            hi = make_uint4(scale_bf16x2(hi.x, factor), scale_bf16x2(hi.y, factor), scale_bf16x2(hi.z, factor), scale_bf16x2(hi.w, factor));
         }
     }
     *reinterpret_cast<uint4 *>(tile + c * 1024 + rr * 16) = lo;
@@ -91,8 +113,12 @@ __global__ __launch_bounds__(256) void pack_cotangent_kernel(const uint16_t * __
 
 hipError_t launch_pack_cotangent(const uint16_t * grad, const uint16_t * grad_second, uint8_t * packed,
                                  uint8_t * packed_second, int rows, int out_features, hipStream_t stream,
-                                 const TaskBuild * build) {
+                                 const TaskBuild * build, const int64_t * gather, const float * scale,
+                                 int64_t gather_rows) {
     if ((grad_second == nullptr) != (packed_second == nullptr)) {
+        return hipErrorInvalidValue;
+    }
+    if (gather != nullptr && (grad_second != nullptr || scale == nullptr || gather_rows <= 0)) {
         return hipErrorInvalidValue;
     }
     const int n_chunks = cotangent_chunks(out_features);
@@ -100,7 +126,8 @@ hipError_t launch_pack_cotangent(const uint16_t * grad, const uint16_t * grad_se
                     grad_second != nullptr ? 2 : 1);
     const ProfileScope scope(6, stream);
     pack_cotangent_kernel<<<grid, 256, 0, stream>>>(grad, grad_second, packed, packed_second, rows, out_features,
-                                                    n_chunks, build != nullptr ? *build : no_task_build());
+                                                    n_chunks, build != nullptr ? *build : no_task_build(), gather,
+                                                    scale, gather_rows);
     return hipGetLastError();
 }
 

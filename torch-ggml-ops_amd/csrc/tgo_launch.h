@@ -182,10 +182,12 @@ static inline int64_t cotangent_workspace_bytes(int64_t rows, int64_t out_featur
     return pad_rows(rows) / 32 * cotangent_chunks(out_features) * 1024;
 }
 // One launch packs one cotangent or both of a pair (`grad_second`/`packed_second` null or set together) and, with
-// `build` set, writes the tile-task list on the side.
+// `build` set, writes the tile-task list on the side.  With `gather` set (single cotangent), packed row r is
+// bf16(scale[r] * grad[gather[r], :]) with `grad` holding `gather_rows` rows; an index outside them gives zeros.
 hipError_t launch_pack_cotangent(const uint16_t * grad, const uint16_t * grad_second, uint8_t * packed,
                                  uint8_t * packed_second, int rows, int out_features, hipStream_t stream,
-                                 const TaskBuild * build = nullptr);
+                                 const TaskBuild * build = nullptr, const int64_t * gather = nullptr,
+                                 const float * scale = nullptr, int64_t gather_rows = 0);
 // `cotangent_*` are buffers written by launch_pack_cotangent.
 // `partial` (dense calls): dense_grad_partial_bytes() of scratch for the split reduction, or nullptr.
 hipError_t launch_mmq_grad_input(const uint8_t * cotangent_first, const uint8_t * cotangent_second,

@@ -47,6 +47,7 @@ lib.tgo_grouped_mmq_forward_gathered.argtypes = [_p, _p, _i64, _p, _p, _p, _p, _
 lib.tgo_grouped_mmq_swiglu.argtypes = [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
 lib.tgo_moe_combine.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]
 lib.tgo_grouped_mmq_grad_input.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
+lib.tgo_grouped_mmq_grad_input_weighted.argtypes = [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
 lib.tgo_profile_enable.argtypes = [_int]
 lib.tgo_profile_read.argtypes = [_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]
 
@@ -76,6 +77,7 @@ EXPORTS = (
     "tgo_grouped_mmq_swiglu",
     "tgo_moe_combine",
     "tgo_grouped_mmq_grad_input",
+    "tgo_grouped_mmq_grad_input_weighted",
     "tgo_profile_enable",
     "tgo_profile_read",
 )

@@ -141,7 +141,10 @@ def measure_decode(args, device) -> dict:
     dense = [synth.random_packed_weight(synth.Q3_K, (4096,), 2048, 20 + i, device=device) for i in range(96)]
     generator = torch.Generator(device=device).manual_seed(5)
     report = {}
+    cases = set(args.decode_cases.split(","))
     for tokens in (1, 4, 8):
+        if f"T{tokens}" not in cases:
+            continue
         routings = []
         for variant in range(8):
             token_of_row, indices, offsets, _ = synth.zipf_routing(tokens, experts, top_k, 100 * tokens + variant, device=device)
@@ -197,29 +200,32 @@ def measure_decode(args, device) -> dict:
             "GBps_gemv_kernels": weight_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
         }
     x = torch.randn(1, 2048, device=device, generator=generator).to(torch.bfloat16)
-    for i in range(args.warmup):
+    if "dense" not in cases:
+        dense = []
+    for i in range(args.warmup if dense else 0):
         tgo.mmq(x, dense[i % 96], synth.Q3_K, 4096)
     torch.cuda.synchronize()
     _native.lib.tgo_profile_enable(1)
     start = time.perf_counter()
-    for i in range(args.steps * 4):
+    for i in range(args.steps * 4 if dense else 0):
         tgo.mmq(x, dense[i % 96], synth.Q3_K, 4096)
     torch.cuda.synchronize()
     elapsed = time.perf_counter() - start
     kernel_ms, launches = _native.profile_read("forward_gemv")
     _native.lib.tgo_profile_enable(0)
     dense_bytes = 4096 * 8 * 110
-    report["dense_Q3_K_M1"] = {
-        "weight_MB": dense_bytes / 1e6,
-        "us_per_call": elapsed / (args.steps * 4) * 1e6,
-        "gemv_kernel_us": kernel_ms / launches * 1e3,
-        "GBps_gemv_kernel": dense_bytes / (kernel_ms / launches * 1e-3) / 1e9,
-    }
+    if launches:
+        report["dense_Q3_K_M1"] = {
+            "weight_MB": dense_bytes / 1e6,
+            "us_per_call": elapsed / (args.steps * 4) * 1e6,
+            "gemv_kernel_us": kernel_ms / launches * 1e3,
+            "GBps_gemv_kernel": dense_bytes / (kernel_ms / launches * 1e-3) / 1e9,
+        }
     # a matrix large enough for bandwidth to matter: one FFN projection of a 70B-class dense model, M = 1, 2, 8, 16
     big_n, big_k = 28672, 8192
-    big = [synth.random_packed_weight(synth.Q4_K, (big_n,), big_k, 40 + i, device=device) for i in range(3)]
+    big = [synth.random_packed_weight(synth.Q4_K, (big_n,), big_k, 40 + i, device=device) for i in range(3)] if "big" in cases else []
     big_bytes = big_n * (big_k // 256) * 144
-    for m in (1, 2, 8, 16):
+    for m in (1, 2, 8, 16) if big else ():
         xb = torch.randn(m, big_k, device=device, generator=generator).to(torch.bfloat16)
         for i in range(args.warmup):
             tgo.mmq(xb, big[i % 3], synth.Q4_K, big_n)
@@ -573,6 +579,9 @@ def main() -> None:
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
     parser.add_argument("--no-cpu-baseline", action="store_true")
+    parser.add_argument("--decode-cases", default="T1,T4,T8,dense,big",
+                        help="decode workload: which cases to run (T1, T4, T8: MoE layer calls; dense: Q3_K [4096,2048] "
+                        "single row; big: Q4_K [28672,8192] with 1..16 rows)")
     parser.add_argument("--no-sub-records", action="store_true",
                         help="pair workload only: skip the down-projection and decode sub-records")
     parser.add_argument("--workload", choices=("pair", "decode", "multi", "gathered", "layer", "dense", "down"), default="pair")

@@ -74,6 +74,8 @@ def test_q8_1_quantizer_matches_oracle_bit_for_bit(ops, oracle, rows, k):
     _, native, _ = ops
     x = random_bf16((rows, k), seed=7 + rows, scale=2.0)
     x[0, :32] = 0  # a zero block
+    # exact halves (scale 127/amax = 1): roundf sends them away from zero; and values that round to -0
+    x[0, 32:64] = torch.tensor([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, -63.5, 126.5, -126.5, -0.25, 0.25, -0.0, 3.5, -3.5] * 2)
     workspace = torch.empty(native.lib.tgo_q8_workspace_bytes(rows, k), dtype=torch.uint8, device="cuda")
     native.check(native.lib.tgo_quantize_q8_1(x.data_ptr(), workspace.data_ptr(), rows, k, None))
     q = torch.empty(rows, k, dtype=torch.int8, device="cuda")

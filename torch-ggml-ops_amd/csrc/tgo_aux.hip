@@ -69,12 +69,24 @@ hipError_t launch_dequant_bf16(const uint8_t * packed, uint16_t * out, int64_t r
 // One workgroup handles 32 rows x 256 values and writes one contiguous 8 KiB run of fragment-ordered int8.
 // Eight consecutive values of a 32-value block per lane (four neighbouring lanes hold the block): the block's
 // scale, the lane's eight int8 values and the block's sum, the same on all four lanes.
-TGO_DEVICE void quantize_eight(const float (&x)[8], uint32_t (&packed)[2], float & d, float & total) {
-    float amax = 0.0f;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        amax = fmaxf(amax, fabsf(x[i]));
-    }
+// round(v) to the nearest integer, halves away from zero (roundf), of a magnitude: the hardware's
+// round-to-nearest-with-ties-up conversion of |v| is exactly that for non-negative inputs.
+TGO_DEVICE int round_magnitude(float v) {
+    int magnitude;
+    asm("v_cvt_rpi_i32_f32 %0, |%1|" : "=v"(magnitude) : "v"(v));
+    return magnitude;
+}
+
+// `bits` are the lane's eight bf16 values as loaded (two per word), `x` the same as floats.  The quants are
+// formed as magnitudes, two per register as 16-bit integers, and get their signs from the bf16 words themselves
+// (an arithmetic shift of each half by 15 is the sign mask of the value it holds): (m ^ s) - s with packed 16-bit
+// operations, then one byte permute per four values.
+typedef short short2_t __attribute__((ext_vector_type(2)));
+TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (&packed)[2], float & d, float & total) {
+    float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fabsf(x[2]));
+    amax = fmaxf(fmaxf(amax, fabsf(x[3])), fabsf(x[4]));
+    amax = fmaxf(fmaxf(amax, fabsf(x[5])), fabsf(x[6]));
+    amax = fmaxf(amax, fabsf(x[7]));
     amax = fmaxf(amax, __shfl_xor(amax, 1));
     amax = fmaxf(amax, __shfl_xor(amax, 2));
 
@@ -88,13 +100,18 @@ TGO_DEVICE void quantize_eight(const float (&x)[8], uint32_t (&packed)[2], float
 
     d = amax == 0.0f ? 0.0f : amax / 127.0f;
     const float d_inv = amax == 0.0f ? 0.0f : 127.0f / amax;
-    packed[0] = 0;
-    packed[1] = 0;
+    const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
+    uint32_t signed_pairs[4];
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int value = static_cast<int>(roundf(x[i] * d_inv));
-        packed[i >> 2] |= static_cast<uint32_t>(value & 0xff) << (8 * (i & 3));
+    for (int pair = 0; pair < 4; ++pair) {
+        const short2_t magnitudes = __builtin_amdgcn_cvt_pk_i16(round_magnitude(x[2 * pair] * d_inv),
+                                                                round_magnitude(x[2 * pair + 1] * d_inv));
+        const short2_t sign = __builtin_bit_cast(short2_t, words[pair]) >> 15;
+        signed_pairs[pair] = __builtin_bit_cast(uint32_t, static_cast<short2_t>((magnitudes ^ sign) - sign));
     }
+    // low byte of each 16-bit half: bytes 0 and 2 of the first word, then of the second
+    packed[0] = __builtin_amdgcn_perm(signed_pairs[1], signed_pairs[0], 0x06040200u);
+    packed[1] = __builtin_amdgcn_perm(signed_pairs[3], signed_pairs[2], 0x06040200u);
 }
 
 TGO_DEVICE void unpack_bf16x8(const uint4 bits, float (&x)[8]) {
@@ -125,13 +142,15 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
         source = gather[row];
         present = source >= 0 && source < input_rows;
     }
-    float x[8] = {};
+    uint4 bits = make_uint4(0, 0, 0, 0);
     if (present) {
-        unpack_bf16x8(*reinterpret_cast<const uint4 *>(input + source * in_features + k), x);
+        bits = *reinterpret_cast<const uint4 *>(input + source * in_features + k);
     }
+    float x[8];
+    unpack_bf16x8(bits, x);
     uint32_t packed[2];
     float d, total;
-    quantize_eight(x, packed, d, total);
+    quantize_eight(bits, x, packed, d, total);
     *reinterpret_cast<uint2 *>(q_out + static_cast<int64_t>(row) * in_features + k) = make_uint2(packed[0], packed[1]);
     if ((threadIdx.x & 3) == 0) {
         const int64_t block = static_cast<int64_t>(row) * (in_features / 32) + k / 32;
@@ -189,10 +208,11 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
     for (int pass = 0; pass < 4; ++pass) {
         const int rr = (tid >> 5) + 8 * pass;
         float x[8];
-        unpack_bf16x8(present[pass] ? bits[pass] : uint4{0, 0, 0, 0}, x);
+        const uint4 row_bits = present[pass] ? bits[pass] : uint4{0, 0, 0, 0};
+        unpack_bf16x8(row_bits, x);
         uint32_t packed[2];
         float d, total;
-        quantize_eight(x, packed, d, total);
+        quantize_eight(row_bits, x, packed, d, total);
         const int half = quarter >> 1;
         uint2 * dst = reinterpret_cast<uint2 *>(tile + block * 1024 + (rr + 32 * half) * 16 + 8 * (quarter & 1));
         *dst = make_uint2(packed[0], packed[1]);

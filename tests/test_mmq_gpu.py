@@ -145,6 +145,30 @@ def test_grad_input_of_small_calls_splits_the_reduction(ops, oracle, qname, rows
     assert not f32(picked)[: rows - 1].any()
 
 
+@pytest.mark.parametrize("qname", ("Q3_K", "Q6_K", "IQ2_S"))
+@pytest.mark.parametrize("rows,n,k", [(70, 136, 768), (300, 136, 768), (70, 37, 768), (300, 72, 1280)])
+def test_blocks_at_every_even_misalignment(ops, oracle, qname, rows, n, k):
+    """Blocks of 110, 210 and 82 bytes start at every even offset inside the 16-byte units the kernels fetch them in.
+    With K = 768 or 1280 a weight row is 2 (mod 4) bytes long, so that offset also changes from row to row; 37 rows of
+    such a weight do not end on a unit boundary, which selects the 2-byte copy instead.  Forward against the oracle,
+    grad-input against the oracle, and a one-hot cotangent returns a weight row bit for bit."""
+    tgo, _, synth = ops
+    qtype = QTYPES[qname]
+    host, device = _weight(synth, qtype, n, k, seed=2468 + qtype)
+    x = random_bf16((rows, k), seed=97)
+    actual = tgo.mmq(x, device, qtype, n)
+    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k))
+    grad_output = random_bf16((rows, n), seed=98)
+    grad = torch.ops.torch_ggml_ops.mmq_grad_input.default(grad_output, device, qtype, k)
+    assert_matches_f32_reference(grad, oracle.grad_input(qtype, bits(grad_output), host.numpy(), n, k), accumulate_noise=2e-6)
+    logical = oracle.bf16_to_f32(oracle.dequant_bf16(qtype, host.numpy(), k))
+    for column in (0, n // 2 + 1, n - 1):
+        one_hot = torch.zeros(rows, n, device="cuda", dtype=torch.bfloat16)
+        one_hot[rows - 1, column] = 1
+        picked = torch.ops.torch_ggml_ops.mmq_grad_input.default(one_hot, device, qtype, k)
+        np.testing.assert_array_equal(f32(picked)[rows - 1], logical[column])
+
+
 @pytest.mark.parametrize("qname", tuple(QTYPES))
 @pytest.mark.parametrize("rows,n", [(10, 37), (129, 64), (260, 200)])
 def test_grad_input_is_logical_weight_jacobian(ops, oracle, qname, rows, n):

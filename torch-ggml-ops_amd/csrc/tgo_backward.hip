@@ -213,7 +213,10 @@ TGO_DEVICE void task_segment(const BackwardArgs & a, int & first, int & tasks) {
 // rows and one 32-column slice of the tile (8 instead of 32 matrix instructions per step, spread over all four
 // SIMDs, 32 accumulator registers instead of 128), and with the smaller register footprint three workgroups share
 // a CU, so that one's barriers and memory waits are covered by another's decoding.
-template <int TYPE, bool SHORT>
+// WIDE (formats whose blocks are not multiples of 16 bytes, when wide_stage_ok holds): a step's packed blocks are
+// requested as aligned 16-byte units while the previous step multiplies, like those of Q4_K / Q5_K, instead of
+// being copied two bytes at a time between the multiplications and the decoding.
+template <int TYPE, bool SHORT, bool WIDE>
 #ifndef TGO_SHORT_OCC
 #define TGO_SHORT_OCC 3
 #endif
@@ -226,7 +229,13 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
     constexpr bool FAST_K45 = TYPE == Q4_K || TYPE == Q5_K;
     constexpr int RAW_UNITS = F::BLOCK_BYTES / 16;                              // 16-byte units per block (fast types)
     constexpr int RAW_REGS = (BWD_NS * RAW_UNITS + BWD_THREADS - 1) / BWD_THREADS;  // units in flight per thread
-    __shared__ __attribute__((aligned(16))) uint8_t raw[BWD_NS * F::RAW_PITCH];
+    static_assert(!(WIDE && FAST_K45), "the wide copy is for the 2-byte aligned formats");
+    using W = WideStage<TYPE>;
+    constexpr int WIDE_REGS = WIDE ? W::template regs<BWD_NS, BWD_THREADS>() : 1;
+    constexpr int SLOT_PITCH = WIDE ? W::PITCH : F::RAW_PITCH;
+    constexpr int SLOT_FRONT = WIDE ? W::FRONT : F::RAW_SHIFT;
+    constexpr bool AHEAD = FAST_K45 || WIDE;   // the packed blocks of the next step travel through registers
+    __shared__ __attribute__((aligned(16))) uint8_t raw[BWD_NS * SLOT_PITCH];
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
     __shared__ float2 scale_min[FAST_K45 ? 4 * (BWD_NS + 8) : 1];
     __shared__ uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
@@ -296,6 +305,7 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
 
     uint4 afrag[2][4] = {};     // cotangent fragments of the step about to be multiplied
     u32x4 raw_regs[FAST_K45 ? RAW_REGS : 1];   // (a native vector type: arrays of the uint4 struct end up in scratch memory)
+    WideRegs<WIDE_REGS> wide_regs;
 
     // requests the cotangent fragments of a step: chunk s covers columns n0 + 16 s .. + 16
     auto load_cotangent = [&](int step) __attribute__((always_inline)) {
@@ -334,11 +344,21 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                         weights + src_row * a.row_bytes + static_cast<int64_t>(kb) * F::BLOCK_BYTES + unit * 16);
                 }
             }
+        } else if constexpr (WIDE) {
+            wide_fetch<TYPE, BWD_NS, BWD_THREADS, WIDE_REGS>(wide_regs, weights + n0 * a.row_bytes, static_cast<int>(a.row_bytes),
+                                                             min(BWD_NS, n_total - n0), kb, tid);
         } else {
             stage_blocks<TYPE>(raw, weights, a.row_bytes, n0, n_total, kb, BWD_NS, tid, BWD_THREADS);
         }
     };
-    auto store_raw = [&]() __attribute__((always_inline)) {
+    auto store_raw = [&](int step) __attribute__((always_inline)) {
+        if constexpr (WIDE) {
+            const int source = step / steps_per_source;
+            const int n0 = (step - source * steps_per_source) * BWD_NS;
+            const uint8_t * weights = a.packed[source] + static_cast<int64_t>(expert) * a.bytes_per_expert;
+            wide_park<TYPE, BWD_NS, BWD_THREADS, WIDE_REGS>(raw, wide_regs, weights + n0 * a.row_bytes, static_cast<int>(a.row_bytes),
+                                                            min(BWD_NS, n_total - n0), kb, tid);
+        }
         if constexpr (FAST_K45) {
 #pragma unroll
             for (int i = 0; i < RAW_REGS; ++i) {
@@ -375,7 +395,7 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                 const int n = id & 63;
                 const int unit = id >> 6;
                 float w[16];
-                decode16_f32<TYPE>(raw + n * F::RAW_PITCH + F::RAW_SHIFT, 8 * half_block + unit, grid, w);
+                decode16_f32<TYPE>(raw + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, w);
                 const bool valid = n0 + n < n_total;
                 // Neighbouring lanes hold neighbouring weight rows of the same 16 values of K.  They swap pairs of
                 // bf16 values so that the even lane writes both rows of an even k and the odd lane both rows of the
@@ -490,13 +510,13 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
         if (wave_active) {
             load_cotangent(step_begin);
         }
-        store_raw();
+        store_raw(step_begin);
         decode(step_begin, wb[0]);
 
         for (int step = step_begin; step < step_end; ++step) {
             const bool more = step + 1 < step_end;
             if (more) {
-                if constexpr (FAST_K45) {
+                if constexpr (AHEAD) {
                     load_raw(step + 1);      // in flight during the MFMAs below
                 }
             }
@@ -524,8 +544,8 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                 if (wave_active) {
                     load_cotangent(step + 1);   // in flight while the next tile is decoded
                 }
-                if constexpr (FAST_K45) {
-                    store_raw();
+                if constexpr (AHEAD) {
+                    store_raw(step + 1);
                 } else {
                     load_raw(step + 1);
                 }
@@ -1382,6 +1402,20 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
         return hipErrorInvalidValue;
     }
     const ProfileScope scope(3, stream);
+    // the general kernel, in its variant for short tasks or not, with the packed blocks fetched as wide units
+    // where the format needs that and the weights allow it
+    const auto general = [&](auto short_tag, dim3 grid, const BackwardArgs & launch_args) {
+        constexpr bool SHORT = decltype(short_tag)::value;
+        if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
+            const int64_t weight_bytes = static_cast<int64_t>(args.out_features) * args.row_bytes;
+            if (wide_stage_ok(args.packed[0], weight_bytes) &&
+                (args.packed[1] == nullptr || wide_stage_ok(args.packed[1], weight_bytes))) {
+                mmq_grad_input_kernel<TYPE, SHORT, true><<<grid, BWD_THREADS, 0, stream>>>(launch_args);
+                return;
+            }
+        }
+        mmq_grad_input_kernel<TYPE, SHORT, false><<<grid, BWD_THREADS, 0, stream>>>(launch_args);
+    };
     if (args.segment == 1) {
         // grouped call: the short tasks (a separate segment of the task list) run in a launch of their own
         BackwardArgs short_args = args;
@@ -1396,7 +1430,7 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
             }
         }
         if (!launched) {
-            mmq_grad_input_kernel<TYPE, true><<<static_cast<unsigned>(total_short), BWD_THREADS, 0, stream>>>(short_args);
+            general(std::true_type{}, dim3(static_cast<unsigned>(total_short)), short_args);
         }
         const hipError_t status = hipGetLastError();
         if (status != hipSuccess) {
@@ -1406,7 +1440,7 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
     if (args.n_splits > 1) {
         // (every format takes the general kernel here: what this path needs is many short workgroups)
         const dim3 grid(static_cast<unsigned>(total), static_cast<unsigned>(args.n_splits));
-        mmq_grad_input_kernel<TYPE, false><<<grid, BWD_THREADS, 0, stream>>>(args);
+        general(std::false_type{}, grid, args);
         const int64_t count = static_cast<int64_t>(args.rows) * args.in_features;
         reduce_partials_kernel<<<static_cast<unsigned>((count / 8 + 255) / 256), 256, 0, stream>>>(
             args.partial, args.dx, count, args.n_splits);
@@ -1426,7 +1460,7 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
             return hipGetLastError();
         }
     }
-    mmq_grad_input_kernel<TYPE, false><<<static_cast<unsigned>(total), BWD_THREADS, 0, stream>>>(args);
+    general(std::false_type{}, dim3(static_cast<unsigned>(total)), args);
     return hipGetLastError();
 }
 

@@ -270,6 +270,92 @@ TGO_DEVICE void stage_blocks(uint8_t * raw, const uint8_t * weights, int64_t row
     }
 }
 
+// ---- register-staged copy for the formats whose blocks are only 2-byte aligned (Q3_K, Q6_K, IQ2_S) ------------
+// stage_blocks moves such blocks two bytes per load, issued where the data is needed.  A block can instead be
+// fetched as the 16-byte aligned units of memory that cover it, a whole reduction step ahead, into registers.  A
+// block then starts m = (its address) % 16 bytes into its first unit, an even number that differs from row to
+// row.  On the way to LDS the odd part of that (m & 2) is taken out with a byte alignment of neighbouring words
+// (each unit carries the first word of the next one for this), the rest (m & 12) by where the words are
+// written, so that the block's first byte lands on the 4-byte aligned position FRONT of its slot and every field
+// the unpackers read as words is aligned.  The up to 12 bytes in front of a block and the bytes behind it that
+// come along land in the slot's own padding.  Units that lie entirely behind the block are not fetched (the lane
+// repeats unit 0).  The first unit starts at or after the 16-byte aligned start of the weight tensor and the
+// last one ends at or before its end rounded up to 16: wide_stage_ok() says when both lie inside the tensor.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+
+template <int TYPE>
+struct WideStage {
+    static constexpr int BLOCK = Format<TYPE>::BLOCK_BYTES;
+    static constexpr int UNITS = (BLOCK + 14 + 15) / 16;       // units that cover a block at any even misalignment
+    static constexpr int FRONT = 12;                           // slot offset of the block's first byte
+    static constexpr int SPAN = FRONT + 16 * UNITS;            // bytes a slot may receive
+    static constexpr int PITCH = (SPAN / 4) % 2 == 1 ? SPAN : SPAN + 4;   // 4 * odd: rows spread over the banks
+    static constexpr int RECIPROCAL = (65536 + UNITS - 1) / UNITS;        // id -> id / UNITS, exact below 3000
+    template <int NROWS, int THREADS>
+    static constexpr int regs() { return (NROWS * UNITS + THREADS - 1) / THREADS; }
+};
+
+// Whether the tensor of one expert may be read in whole aligned units: its first and last byte are unit
+// boundaries (the bytes of an expert end where the next expert's begin, so this covers stacked experts).
+static __host__ __device__ inline bool wide_stage_ok(const void * packed, int64_t bytes_per_expert) {
+    return (reinterpret_cast<uintptr_t>(packed) & 15) == 0 && (bytes_per_expert & 15) == 0;
+}
+
+template <int REGS>
+struct WideRegs {
+    u32x4_t unit[REGS];
+    uint32_t next[REGS];   // first word of the following unit
+};
+
+// `tile`: first byte of weight row 0 of the tile (wave-uniform); rows past rows_valid - 1 repeat the last valid
+// row.  (rows_valid * row_bytes + the bytes of a row) must stay below 2^31.
+template <int TYPE, int NROWS, int THREADS, int REGS>
+TGO_DEVICE void wide_fetch(WideRegs<REGS> & regs, const uint8_t * tile, int row_bytes, int rows_valid, int kb, int t) {
+    using W = WideStage<TYPE>;
+    static_assert(NROWS * W::UNITS < 3000, "range of the reciprocal");
+    const uint32_t tile_m = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) & 15u;
+    const uint8_t * const aligned = tile - tile_m;
+    const uint32_t column = tile_m + static_cast<uint32_t>(kb) * W::BLOCK;
+#pragma unroll
+    for (int i = 0; i < REGS; ++i) {
+        const int id = min(t + THREADS * i, NROWS * W::UNITS - 1);
+        const int row = static_cast<int>(__umul24(id, W::RECIPROCAL) >> 16);
+        int unit = id - row * W::UNITS;
+        const uint32_t first = __umul24(min(row, rows_valid - 1), row_bytes) + column;   // of the block, from `aligned`
+        const int reach = static_cast<int>(first & 15u) + W::BLOCK;                      // block end, from its first unit
+        const bool carries = 16 * (unit + 1) < reach;   // the following unit still holds bytes of the block
+        unit = 16 * unit < reach ? unit : 0;
+        const uint32_t offset = (first & ~15u) + 16u * unit;
+        regs.unit[i] = *reinterpret_cast<const u32x4_t *>(aligned + offset);
+        regs.next[i] = carries ? *reinterpret_cast<const uint32_t *>(aligned + offset + 16) : 0u;
+    }
+}
+
+// Writes what wide_fetch brought (same arguments) into slots of WideStage::PITCH bytes; the block of row r then
+// starts at raw + r * PITCH + FRONT.
+template <int TYPE, int NROWS, int THREADS, int REGS>
+TGO_DEVICE void wide_park(uint8_t * raw, const WideRegs<REGS> & regs, const uint8_t * tile, int row_bytes,
+                          int rows_valid, int kb, int t) {
+    using W = WideStage<TYPE>;
+    const uint32_t column = (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) & 15u) + static_cast<uint32_t>(kb) * W::BLOCK;
+#pragma unroll
+    for (int i = 0; i < REGS; ++i) {
+        const int id = t + THREADS * i;
+        if (id < NROWS * W::UNITS) {
+            const int row = static_cast<int>(__umul24(id, W::RECIPROCAL) >> 16);
+            const int unit = id - row * W::UNITS;
+            const uint32_t m = (__umul24(min(row, rows_valid - 1), row_bytes) + column) & 15u;
+            const uint32_t shift = m & 2u;
+            const u32x4_t d = regs.unit[i];
+            uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * W::PITCH + W::FRONT - (m & 12u) + 16 * unit);
+            dst[0] = __builtin_amdgcn_alignbyte(d.y, d.x, shift);
+            dst[1] = __builtin_amdgcn_alignbyte(d.z, d.y, shift);
+            dst[2] = __builtin_amdgcn_alignbyte(d.w, d.z, shift);
+            dst[3] = __builtin_amdgcn_alignbyte(regs.next[i], d.w, shift);
+        }
+    }
+}
+
 TGO_DEVICE uint32_t lds_u32(const uint8_t * p) { return *reinterpret_cast<const uint32_t *>(p); }
 TGO_DEVICE uint32_t lds_u16(const uint8_t * p) { return *reinterpret_cast<const uint16_t *>(p); }
 

@@ -69,12 +69,15 @@ struct ForwardArgs {
     int swiglu;        // 1: a workgroup runs gate (-> y) then up and stores swiglu(gate, up) -> y_second
     int task_slots;
     int dense_row_tile;   // dense calls: rows per workgroup (the format's row tile, or 32 when that fills the chip better)
+    int wide;             // 2-byte aligned formats: the weights may be fetched as aligned 16-byte units (wide_stage_ok)
 };
 
 // LDS of one workgroup.
 template <int TYPE>
 struct ForwardLds {
-    alignas(16) uint8_t raw[FWD_TN * Format<TYPE>::RAW_PITCH];        // packed blocks of one super-block column
+    static constexpr int RAW_SLOT = Format<TYPE>::BLOCK_BYTES % 16 == 0 || Format<TYPE>::RAW_PITCH > WideStage<TYPE>::PITCH
+                                        ? Format<TYPE>::RAW_PITCH : WideStage<TYPE>::PITCH;
+    alignas(16) uint8_t raw[FWD_TN * RAW_SLOT];                        // packed blocks of one super-block column
     alignas(16) uint8_t wq[Format<TYPE>::PLANES][FWD_TN * 256];        // int8 weight operand in fragment order
     alignas(16) float ws[8][FWD_TN];                                   // block scales
     alignas(16) float wm[Format<TYPE>::HAS_MIN ? 8 : 1][FWD_TN];       // block minima
@@ -82,7 +85,9 @@ struct ForwardLds {
     uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
 };
 
-template <int TYPE, bool NARROW>
+// WIDE (formats whose blocks are not multiples of 16 bytes): the packed blocks are prefetched into registers as
+// aligned units like those of Q4_K / Q5_K (wide_fetch) instead of being copied two bytes at a time when needed.
+template <int TYPE, bool NARROW, bool WIDE>
 TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int n_tile, bool second, int expert,
                              int row_start, int row_end) {
     using F = Format<TYPE>;
@@ -141,6 +146,12 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
     constexpr int RAW_UNITS = RAW_IN_REGS ? F::BLOCK_BYTES / 16 : 1;
     constexpr int RAW_REGS = RAW_IN_REGS ? (FWD_TN * RAW_UNITS + THREADS - 1) / THREADS : 1;
     uint4 raw_next[RAW_REGS];
+    static_assert(!(WIDE && RAW_IN_REGS), "the wide copy is for the 2-byte aligned formats");
+    using W = WideStage<TYPE>;
+    constexpr int WIDE_REGS = WIDE ? W::template regs<FWD_TN, THREADS>() : 1;
+    WideRegs<WIDE_REGS> wide_next;
+    constexpr int SLOT_PITCH = WIDE ? W::PITCH : F::RAW_PITCH;
+    constexpr int SLOT_FRONT = WIDE ? W::FRONT : F::RAW_SHIFT;
     // (`t` is the thread id: the main loop passes a copy the compiler cannot see through, so that the small
     // address computations below are redone per round instead of being kept alive, and spilled, across it)
     // (unit id -> weight row by a 24-bit multiply and a shift, exact for the few thousand ids of a tile)
@@ -158,6 +169,8 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
                 const uint32_t offset = __umul24(min(row, tile_rows - 1), static_cast<uint32_t>(a.row_bytes)) + unit * 16;
                 raw_next[i] = *reinterpret_cast<const uint4 *>(base + offset);
             }
+        } else if constexpr (WIDE) {
+            wide_fetch<TYPE, FWD_TN, THREADS, WIDE_REGS>(wide_next, tile_weights, static_cast<int>(a.row_bytes), tile_rows, kb, t);
         }
     };
     auto store_raw = [&](int kb, int t) {
@@ -170,6 +183,8 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
                 uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
                 dst[0] = raw_next[i].x; dst[1] = raw_next[i].y; dst[2] = raw_next[i].z; dst[3] = raw_next[i].w;
             }
+        } else if constexpr (WIDE) {
+            wide_park<TYPE, FWD_TN, THREADS, WIDE_REGS>(raw, wide_next, tile_weights, static_cast<int>(a.row_bytes), tile_rows, kb, t);
         } else {
             stage_blocks<TYPE>(raw, weights, a.row_bytes, n0, a.out_features, kb, FWD_TN, t, THREADS);
         }
@@ -267,7 +282,7 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
             constexpr int UNIT_STEP = THREADS / FWD_TN;
             const uint32_t row = static_cast<uint32_t>(t) & (FWD_TN - 1);
             const uint32_t first_unit = static_cast<uint32_t>(t) / FWD_TN;
-            const uint8_t * blk = raw + row * F::RAW_PITCH + F::RAW_SHIFT;
+            const uint8_t * blk = raw + row * SLOT_PITCH + SLOT_FRONT;
             const uint32_t row_slot = ((row >> 5) * 8 * 64 + (row & 31)) * 16;
             if constexpr ((TYPE == Q4_K || TYPE == Q5_K) && UNIT_STEP == 2) {
                 // The thread's units are the same 16-value half (first_unit) of all eight 32-value groups, so
@@ -492,6 +507,32 @@ TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second,
     return true;
 }
 
+// A task of at most 32 rows has work for one wave only in the usual split (a wave = 32 rows x 128 weight
+// rows).  Such tasks are common under skewed routing, so for them the four waves of a single-plane
+// workgroup take one of the four 32-row weight tiles each instead.  The variants are separate
+// instantiations of the task body so that neither's registers weigh on the other.
+template <int TYPE>
+TGO_DEVICE void forward_any_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int n_tile, bool second, int expert,
+                                 int row_start, int row_end) {
+    constexpr bool SINGLE = Format<TYPE>::PLANES == 1;
+    const bool narrow = SINGLE && row_end - row_start <= 32;
+    if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
+        if (a.wide != 0) {
+            if (narrow) {
+                forward_task<TYPE, SINGLE, true>(a, lds, n_tile, second, expert, row_start, row_end);
+            } else {
+                forward_task<TYPE, false, true>(a, lds, n_tile, second, expert, row_start, row_end);
+            }
+            return;
+        }
+    }
+    if (narrow) {
+        forward_task<TYPE, SINGLE, false>(a, lds, n_tile, second, expert, row_start, row_end);
+    } else {
+        forward_task<TYPE, false, false>(a, lds, n_tile, second, expert, row_start, row_end);
+    }
+}
+
 template <int TYPE>
 __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_kernel(const ForwardArgs a) {
     using F = Format<TYPE>;
@@ -505,15 +546,7 @@ __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_ke
     if (!forward_pick<TYPE>(a, n_tile, second, expert, row_start, row_end)) {
         return;
     }
-    // A task of at most 32 rows has work for one wave only in the usual split (a wave = 32 rows x 128 weight
-    // rows).  Such tasks are common under skewed routing, so for them the four waves of a single-plane
-    // workgroup take one of the four 32-row weight tiles each instead.  The two variants are separate
-    // instantiations of the task body so that neither's registers weigh on the other.
-    if (PLANES == 1 && row_end - row_start <= 32) {
-        forward_task<TYPE, PLANES == 1>(a, lds, n_tile, second, expert, row_start, row_end);
-    } else {
-        forward_task<TYPE, false>(a, lds, n_tile, second, expert, row_start, row_end);
-    }
+    forward_any_task<TYPE>(a, lds, n_tile, second, expert, row_start, row_end);
 }
 
 // Fused SwiGLU, its own kernel so that the plain forward's register allocation is untouched.  The gate tile
@@ -533,11 +566,7 @@ __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_sw
     }
 #pragma unroll 1
     for (int pass = 0; pass < 2; ++pass) {
-        if (PLANES == 1 && row_end - row_start <= 32) {
-            forward_task<TYPE, PLANES == 1>(a, lds, n_tile, pass == 1, expert, row_start, row_end);
-        } else {
-            forward_task<TYPE, false>(a, lds, n_tile, pass == 1, expert, row_start, row_end);
-        }
+        forward_any_task<TYPE>(a, lds, n_tile, pass == 1, expert, row_start, row_end);
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
         __syncthreads();
     }
@@ -576,6 +605,9 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     args.projections = packed_second != nullptr && args.swiglu == 0 ? 2 : 1;
     args.bytes_per_expert = bytes_per_expert;
     args.row_bytes = static_cast<int64_t>(in_features / QK_K) * block_bytes(quant_type);
+    // (a dense call has one "expert": the whole weight)
+    const int64_t weight_bytes = static_cast<int64_t>(out_features) * args.row_bytes;
+    args.wide = wide_stage_ok(packed, weight_bytes) && (packed_second == nullptr || wide_stage_ok(packed_second, weight_bytes)) ? 1 : 0;
     args.qx = ws.q;
     args.dx = ws.d;
     args.sx = ws.sum;

@@ -236,6 +236,7 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
     constexpr int SLOT_FRONT = WIDE ? W::FRONT : F::RAW_SHIFT;
     constexpr bool AHEAD = FAST_K45 || WIDE;   // the packed blocks of the next step travel through registers
     __shared__ __attribute__((aligned(16))) uint8_t raw[BWD_NS * SLOT_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t raw_odd[WIDE ? BWD_NS * SLOT_PITCH : 16];   // second slot of the WIDE pipeline
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
     __shared__ float2 scale_min[FAST_K45 ? 4 * (BWD_NS + 8) : 1];
     __shared__ uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
@@ -503,6 +504,168 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                     }
                 }
             }
+        }
+    } else if constexpr (WIDE) {
+        // One barrier per step, and every wave both multiplies and dequantizes between two barriers: while the matrix
+        // instructions of step i run on tile i % 2, the same wave's vector instructions decode step i + 1 from its
+        // parked blocks into the other tile (the two kinds of instruction issue independently, so inside one block
+        // of code they overlap), the blocks of step i + 2 go from registers to the raw slot that step i was decoded
+        // from, those of step i + 3 are requested, and each quarter of the cotangent fragments is re-requested for
+        // step i + 1 as soon as the matrix instructions of step i that read it have been issued.  Steps past the
+        // end repeat the last one where that avoids a branch around a load.
+        const int last = step_end - 1;
+        auto blocks_of = [&](int step, const uint8_t *& tile_rows, int & rows_valid) __attribute__((always_inline)) {
+            step = min(step, last);
+            const int source = step / steps_per_source;
+            const int n0 = (step - source * steps_per_source) * BWD_NS;
+            tile_rows = a.packed[source] + static_cast<int64_t>(expert) * a.bytes_per_expert + n0 * a.row_bytes;
+            rows_valid = min(BWD_NS, n_total - n0);
+        };
+        auto request = [&](int step) __attribute__((always_inline)) {
+            const uint8_t * tile_rows;
+            int rows_valid;
+            blocks_of(step, tile_rows, rows_valid);
+            wide_fetch<TYPE, BWD_NS, BWD_THREADS, WIDE_REGS>(wide_regs, tile_rows, static_cast<int>(a.row_bytes), rows_valid, kb, tid);
+        };
+        auto park = [&](int step, uint8_t * slot) __attribute__((always_inline)) {
+            const uint8_t * tile_rows;
+            int rows_valid;
+            blocks_of(step, tile_rows, rows_valid);
+            wide_park<TYPE, BWD_NS, BWD_THREADS, WIDE_REGS>(slot, wide_regs, tile_rows, static_cast<int>(a.row_bytes), rows_valid, kb, tid);
+        };
+        // half of a step's 64 rows x 8 units of 16 values; a half-wave writes 32 consecutive n of one k
+        auto decode_pass = [&](int step, int pass, const uint8_t * slot, uint16_t * tile) __attribute__((always_inline)) {
+            const int source = step / steps_per_source;
+            const int n0 = (step - source * steps_per_source) * BWD_NS;
+            const int n = lane;
+            const int unit = wave + 4 * pass;   // (wave-uniform: the unit's shifts and offsets are scalars)
+            float w[16];
+            decode16_f32<TYPE>(slot + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, w);
+            // rows past the end of the weight matrix become zeros (a mask the compiler cannot see through: a visible
+            // condition ends up as a branch around part of the arithmetic, which splits the block of code that the
+            // matrix and vector instructions are meant to share)
+            uint32_t keep = n0 + n < n_total ? 0xffffffffu : 0u;
+            asm volatile("" : "+v"(keep));
+            // (pairs of lanes swap halves so that each writes both rows of one k: see the two-barrier loop's decode)
+            const uint32_t selector = (lane & 1) != 0 ? 0x03020706u : 0x05040100u;
+            uint32_t * const pair_row = reinterpret_cast<uint32_t *>(&tile[(unit * 16 + (lane & 1)) * BWD_PITCH + (n & ~1)]);
+#pragma unroll
+            for (int j = 0; j < 16; j += 2) {
+                const uint32_t own = pack_bf16x2(w[j], w[j + 1]) & keep;
+                const uint32_t other = static_cast<uint32_t>(
+                    __builtin_amdgcn_mov_dpp(static_cast<int>(own), 0xB1, 0xf, 0xf, true));   // lane ^ 1
+                pair_row[j * (BWD_PITCH / 2)] = __builtin_amdgcn_perm(other, own, selector);
+            }
+        };
+        auto request_cotangent = [&](int step, int s) __attribute__((always_inline)) {
+            const int source = step / steps_per_source;
+            const int n0 = (step - source * steps_per_source) * BWD_NS;
+            const uint8_t * base = a.cotangent[source];
+#pragma unroll
+            for (int rt = 0; rt < 2; ++rt) {
+                if (!SHORT || rt < row_tiles) {
+                    // (the packed cotangent is zero padded to whole steps of 64 columns)
+                    afrag[rt][s] = *reinterpret_cast<const uint4 *>(
+                        base + lane_offset[rt] + static_cast<int64_t>((n0 >> 4) + s) * 1024);
+                }
+            }
+        };
+        // the weight fragments of chunk s of a tile (one per 32-column tile of the wave), and the chunk's multiplications
+        uint4 fragment[2][KT];
+        auto read_fragments = [&](const uint16_t * tile, int s) __attribute__((always_inline)) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const int k = (SHORT ? wave : kt) * 32 + l32;
+                fragment[s & 1][kt] = *reinterpret_cast<const uint4 *>(&tile[k * BWD_PITCH + 16 * s + 8 * half]);
+            }
+        };
+        auto multiply = [&](int s) __attribute__((always_inline)) {
+#pragma unroll
+            for (int kt = 0; kt < KT; ++kt) {
+                const v8bf bfrag = __builtin_bit_cast(v8bf, fragment[s & 1][kt]);
+#pragma unroll
+                for (int rt = 0; rt < 2; ++rt) {
+                    if (!SHORT || rt < row_tiles) {
+                        acc[rt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                            __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0);
+                    }
+                }
+            }
+        };
+        request(step_begin);
+        park(step_begin, raw);
+        request(step_begin + 1);
+        __syncthreads();
+        decode_pass(step_begin, 0, raw, wb[0]);
+        decode_pass(step_begin, 1, raw, wb[0]);
+        if (wave_active) {
+#pragma unroll
+            for (int s = 0; s < 4; ++s) {
+                request_cotangent(step_begin, s);
+            }
+        }
+        park(step_begin + 1, raw_odd);
+        request(step_begin + 2);
+        __syncthreads();
+        auto run = [&](auto active_tag) __attribute__((always_inline)) {
+            constexpr bool ACTIVE = decltype(active_tag)::value;
+#ifndef TGO_IL_VALU
+#define TGO_IL_VALU 12
+#endif
+#pragma unroll 1
+            for (int step = step_begin; step < last; ++step) {
+                const int parity = (step - step_begin) & 1;
+                const uint16_t * tile = wb[parity];
+                uint16_t * next_tile = wb[parity ^ 1];
+                const uint8_t * next_raw = parity != 0 ? raw : raw_odd;
+                if constexpr (ACTIVE) {
+                    read_fragments(tile, 0);
+                }
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    if constexpr (ACTIVE) {
+                        if (s + 1 < 4) {
+                            read_fragments(tile, s + 1);   // an LDS round trip ahead of the instructions they feed
+                        }
+                        multiply(s);
+                        request_cotangent(step + 1, s);
+                    }
+                    if (s == 0 || s == 2) {
+                        decode_pass(step + 1, s >> 1, next_raw, next_tile);
+                    }
+                    if (s == 1) {
+                        park(step + 2, parity != 0 ? raw_odd : raw);
+                    }
+                    if (s == 3) {
+                        request(step + 3);
+                    }
+                    if constexpr (ACTIVE && !SHORT && TGO_IL_VALU > 0) {
+                        // one matrix instruction, then a run of the vector instructions that share its chunk
+#pragma unroll
+                        for (int i = 0; i < 2 * KT; ++i) {
+                            __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, TGO_IL_VALU, 0);
+                        }
+                    }
+                }
+                __syncthreads();
+            }
+            if constexpr (ACTIVE) {
+                const uint16_t * tile = wb[(last - step_begin) & 1];
+                read_fragments(tile, 0);
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    if (s + 1 < 4) {
+                        read_fragments(tile, s + 1);
+                    }
+                    multiply(s);
+                }
+            }
+        };
+        if (wave_active) {
+            run(std::true_type{});
+        } else {
+            run(std::false_type{});
         }
     } else {
         // prologue: the first step staged and decoded, its cotangent fragments requested

@@ -327,7 +327,9 @@ TGO_DEVICE void wide_fetch(WideRegs<REGS> & regs, const uint8_t * tile, int row_
         unit = 16 * unit < reach ? unit : 0;
         const uint32_t offset = (first & ~15u) + 16u * unit;
         regs.unit[i] = *reinterpret_cast<const u32x4_t *>(aligned + offset);
-        regs.next[i] = carries ? *reinterpret_cast<const uint32_t *>(aligned + offset + 16) : 0u;
+        // (where nothing of the block follows, the word is never looked at: the lane re-reads its own unit
+        // rather than branching around the load)
+        regs.next[i] = *reinterpret_cast<const uint32_t *>(aligned + offset + (carries ? 16u : 0u));
     }
 }
 
@@ -340,19 +342,18 @@ TGO_DEVICE void wide_park(uint8_t * raw, const WideRegs<REGS> & regs, const uint
     const uint32_t column = (static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) & 15u) + static_cast<uint32_t>(kb) * W::BLOCK;
 #pragma unroll
     for (int i = 0; i < REGS; ++i) {
-        const int id = t + THREADS * i;
-        if (id < NROWS * W::UNITS) {
-            const int row = static_cast<int>(__umul24(id, W::RECIPROCAL) >> 16);
-            const int unit = id - row * W::UNITS;
-            const uint32_t m = (__umul24(min(row, rows_valid - 1), row_bytes) + column) & 15u;
-            const uint32_t shift = m & 2u;
-            const u32x4_t d = regs.unit[i];
-            uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * W::PITCH + W::FRONT - (m & 12u) + 16 * unit);
-            dst[0] = __builtin_amdgcn_alignbyte(d.y, d.x, shift);
-            dst[1] = __builtin_amdgcn_alignbyte(d.z, d.y, shift);
-            dst[2] = __builtin_amdgcn_alignbyte(d.w, d.z, shift);
-            dst[3] = __builtin_amdgcn_alignbyte(regs.next[i], d.w, shift);
-        }
+        // (ids past the tile repeated its last unit in wide_fetch: they write the same words to the same place)
+        const int id = min(t + THREADS * i, NROWS * W::UNITS - 1);
+        const int row = static_cast<int>(__umul24(id, W::RECIPROCAL) >> 16);
+        const int unit = id - row * W::UNITS;
+        const uint32_t m = (__umul24(min(row, rows_valid - 1), row_bytes) + column) & 15u;
+        const uint32_t shift = m & 2u;
+        const u32x4_t d = regs.unit[i];
+        uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * W::PITCH + W::FRONT - (m & 12u) + 16 * unit);
+        dst[0] = __builtin_amdgcn_alignbyte(d.y, d.x, shift);
+        dst[1] = __builtin_amdgcn_alignbyte(d.z, d.y, shift);
+        dst[2] = __builtin_amdgcn_alignbyte(d.w, d.z, shift);
+        dst[3] = __builtin_amdgcn_alignbyte(regs.next[i], d.w, shift);
     }
 }
 
@@ -442,7 +443,7 @@ TGO_DEVICE void unpack16(const uint8_t * blk, int u, const uint2 * grid, int (&q
             }
         }
         const uint8_t * scales = blk + 96;
-        const int low = u < 8 ? scales[u] : scales[u - 8] >> 4;
+        const int low = scales[u & 7] >> (4 * (u >> 3));
         const int high = scales[8 + (u & 3)] >> (2 * (u >> 2));
         sub = ((low & 0x0f) | ((high & 3) << 4)) - 32;
     } else {  // IQ2_S
@@ -491,7 +492,7 @@ TGO_DEVICE void decode16_f32(const uint8_t * blk, int u, const uint2 * grid, flo
                 words[t] = (low & 0x03030303u) | ((high & 0x01010101u) << 2);
             }
             const uint8_t * scales = blk + 96;
-            const int low = u < 8 ? scales[u] : scales[u - 8] >> 4;
+            const int low = scales[u & 7] >> (4 * (u >> 3));
             const int high = scales[8 + (u & 3)] >> (2 * (u >> 2));
             sub = ((low & 0x0f) | ((high & 3) << 4)) - 32;
             d = half_bits_to_float(lds_u16(blk + 108));
@@ -584,7 +585,7 @@ TGO_DEVICE void decode16_int8(const uint8_t * blk, int u, const uint2 * grid, ui
         const int shift_l = 2 * ((i0 & 127) >> 5);
         const int shift_h = i0 >> 5;
         const uint8_t * scales = blk + 96;
-        const int low = u < 8 ? scales[u] : scales[u - 8] >> 4;
+        const int low = scales[u & 7] >> (4 * (u >> 3));
         const int high = scales[8 + (u & 3)] >> (2 * (u >> 2));
         const int sub = ((low & 0x0f) | ((high & 3) << 4)) - 32;
         const uint32_t s = static_cast<uint32_t>(sub < 0 ? -sub : sub);

@@ -188,12 +188,26 @@ def test_role_split_kernel_every_prefetch_phase(ops, oracle, qname, n, sources):
     5 and 8 steps per source, one or two sources and several items per workgroup, every ring phase meets every
     position in an item; a one-hot cotangent per step must return that step's weight row exactly (bit for bit),
     and random cotangents must match the oracle.  Groups of 70..300 rows keep the tasks out of the short-task kernel."""
+    _check_one_hot_and_random_cotangents(ops, oracle, qname, n, sources, [70, 300, 129], [2, 0, 3])
+
+
+@pytest.mark.parametrize("sources", (1, 2))
+@pytest.mark.parametrize("n", (64, 200, 512))
+@pytest.mark.parametrize("qname", ("Q4_K", "Q5_K"))
+def test_short_remainders_next_to_full_tiles(ops, oracle, qname, n, sources):
+    """Remainders of 1, 18, 32 and 33 rows behind full 256-row tiles (groups of 257, 530, 288 and 289 rows), a group
+    of exactly 256 rows and one of 31: the full tiles run in the persistent kernel, the remainders in the short-task
+    kernel, and both write neighbouring rows of one output.  Every row gets a one-hot cotangent that must return a
+    weight row bit for bit, and random cotangents must match the oracle."""
+    _check_one_hot_and_random_cotangents(ops, oracle, qname, n, sources, [257, 31, 288, 256, 289, 530], [1, 3, 0, 2, 5, 4])
+
+
+def _check_one_hot_and_random_cotangents(ops, oracle, qname, n, sources, sizes, experts):
     tgo, synth = ops
     qtype, k = QTYPES[qname], 1024
-    sizes = [70, 300, 129]
-    experts, offsets = [2, 0, 3], np.cumsum(sizes).tolist()
+    offsets = np.cumsum(sizes).tolist()
     rows = offsets[-1]
-    host = [synth.random_packed_weight(qtype, (4, n), k, seed=700 + 10 * s + qtype) for s in range(sources)]
+    host = [synth.random_packed_weight(qtype, (max(experts) + 1, n), k, seed=700 + 10 * s + qtype) for s in range(sources)]
     device = [h.cuda() for h in host]
     metadata = _metadata(experts, offsets)
     op_single = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default

@@ -605,6 +605,87 @@ TGO_DEVICE void decode16_int8(const uint8_t * blk, int u, const uint2 * grid, ui
         }
         return;
     }
+    if constexpr (TYPE == Q6_K) {
+        // Four values per step, as two pairs of 16-bit lanes (bytes 0 and 2, bytes 1 and 3 of a word).  With
+        // b = q + 32 (0..63): t = sc * b + (64 - 32 sc) = sc * q + 64, one packed multiply-add; the low plane is
+        // (t & 127) - 64, of which only the low byte is kept, the high plane t >> 7 (arithmetic), since
+        // sc * q - low = t - (t & 127).  |sc * q| <= 4096, so nothing leaves its 16-bit lane.
+        typedef short pair16 __attribute__((ext_vector_type(2)));
+        typedef unsigned short upair16 __attribute__((ext_vector_type(2)));
+        const int chunk = u >> 3;
+        const int rem = (16 * u) & 127;
+        const uint8_t * ql = blk + chunk * 64 + (rem & 63);
+        const uint8_t * qh = blk + 128 + chunk * 32 + ((16 * u) & 31);
+        const int shift_l = 4 * (rem >> 6);
+        const int shift_h = 2 * ((rem >> 5) & 3);
+        const short sc = static_cast<int8_t>(blk[192 + u]);
+        const short offset = static_cast<short>(64 - 32 * sc);
+        const pair16 scale = {sc, sc};
+        const pair16 shift = {offset, offset};
+        const pair16 mask7 = {127, 127};
+        const pair16 rebias = {192, 192};   // -64 modulo 256: only the low byte of a lane is kept
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t low = lds_u32(ql + 4 * t) >> shift_l;
+            const uint32_t high = lds_u32(qh + 4 * t) >> shift_h;
+            const uint32_t b = (low & 0x0f0f0f0fu) | ((high & 0x03030303u) << 4);
+            const pair16 even = __builtin_bit_cast(pair16, b & 0x00ff00ffu);
+            const pair16 odd = __builtin_bit_cast(pair16, (b >> 8) & 0x00ff00ffu);
+            const pair16 t_even = even * scale + shift;
+            const pair16 t_odd = odd * scale + shift;
+            const uint32_t low_even = __builtin_bit_cast(uint32_t, (t_even & mask7) + rebias);
+            const uint32_t low_odd = __builtin_bit_cast(uint32_t, (t_odd & mask7) + rebias);
+            const uint32_t high_even = __builtin_bit_cast(uint32_t, t_even >> 7);
+            const uint32_t high_odd = __builtin_bit_cast(uint32_t, t_odd >> 7);
+            // bytes (even.0, odd.0, even.2, odd.2)
+            lo[t] = __builtin_amdgcn_perm(low_odd, low_even, 0x06020400u);
+            hi[t] = __builtin_amdgcn_perm(high_odd, high_even, 0x06020400u);
+        }
+        return;
+    }
+    if constexpr (TYPE == IQ2_S) {
+        // The same two-lane arithmetic: the codebook word holds four magnitudes m, p = (2 s + 1) * m <= 1333 is one
+        // packed multiply, the sign bits become lane masks (0 or -1) that negate p as (p ^ mask) - mask, and
+        // t = +-p + 64 splits into the planes as above.
+        typedef short pair16 __attribute__((ext_vector_type(2)));
+        const uint8_t * qs = blk + 2;
+        const uint32_t idx_pair = lds_u16(qs + 2 * u);
+        const int sign_pair = static_cast<int>(lds_u16(qs + 32 + 2 * u));
+        const uint32_t qh = blk[66 + (u >> 1)] >> (4 * (u & 1));
+        const short multiplier = static_cast<short>(2 * ((blk[74 + (u >> 1)] >> (4 * (u & 1))) & 0x0f) + 1);
+        const pair16 scale = {multiplier, multiplier};
+        const pair16 bias = {64, 64};
+        const pair16 mask7 = {127, 127};
+        const pair16 rebias = {192, 192};
+#pragma unroll
+        for (int gsel = 0; gsel < 2; ++gsel) {
+            const uint32_t index = ((idx_pair >> (8 * gsel)) & 0xff) | (((qh >> (2 * gsel)) & 3) << 8);
+            const uint2 word = grid[index];
+#pragma unroll
+            for (int part = 0; part < 2; ++part) {
+                const uint32_t w = part == 0 ? word.x : word.y;
+                const int bit = 8 * gsel + 4 * part;   // sign bit of the word's first value
+                const pair16 even = __builtin_bit_cast(pair16, w & 0x00ff00ffu);
+                const pair16 odd = __builtin_bit_cast(pair16, (w >> 8) & 0x00ff00ffu);
+                // (two sign-extended one-bit fields, low halves side by side)
+                const pair16 mask_even = __builtin_bit_cast(pair16, __builtin_amdgcn_perm(
+                    static_cast<uint32_t>(__builtin_amdgcn_sbfe(sign_pair, bit + 2, 1)),
+                    static_cast<uint32_t>(__builtin_amdgcn_sbfe(sign_pair, bit, 1)), 0x05040100u));
+                const pair16 mask_odd = __builtin_bit_cast(pair16, __builtin_amdgcn_perm(
+                    static_cast<uint32_t>(__builtin_amdgcn_sbfe(sign_pair, bit + 3, 1)),
+                    static_cast<uint32_t>(__builtin_amdgcn_sbfe(sign_pair, bit + 1, 1)), 0x05040100u));
+                const pair16 t_even = ((even * scale) ^ mask_even) - mask_even + bias;
+                const pair16 t_odd = ((odd * scale) ^ mask_odd) - mask_odd + bias;
+                const uint32_t low_even = __builtin_bit_cast(uint32_t, (t_even & mask7) + rebias);
+                const uint32_t low_odd = __builtin_bit_cast(uint32_t, (t_odd & mask7) + rebias);
+                const uint32_t high_even = __builtin_bit_cast(uint32_t, t_even >> 7);
+                const uint32_t high_odd = __builtin_bit_cast(uint32_t, t_odd >> 7);
+                lo[2 * gsel + part] = __builtin_amdgcn_perm(low_odd, low_even, 0x06020400u);
+                hi[2 * gsel + part] = __builtin_amdgcn_perm(high_odd, high_even, 0x06020400u);
+            }
+        }
+        return;
+    }
     int q[16];
     int sub, mn;
     unpack16<TYPE>(blk, u, grid, q, sub, mn);
@@ -676,7 +757,9 @@ TGO_DEVICE uint4 swiglu_bf16x8(const uint4 gate, const uint4 up) {
 // skipped.  Needs a 16-byte aligned dst and row_stride % 8 == 0 for the wide path, else stores 2 bytes each.
 // WIDE_ONLY drops the 2-byte path for callers whose destination always qualifies.
 // With `gate` set (same geometry as dst) the value stored is swiglu(gate element, bf16 of the result).
-template <int PITCH, bool WIDE_ONLY = false, typename V16>
+// TRANSPOSED: the tiles were computed with the operands swapped, so a lane holds row l32 and, as element v of
+// tile t, column 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4 (four neighbouring columns per group of four elements).
+template <int PITCH, bool WIDE_ONLY = false, bool TRANSPOSED = false, typename V16>
 TGO_DEVICE void store_rows_32x128(uint16_t * stage, const V16 (&tiles)[4], uint16_t * dst, int64_t row_stride,
                                   int valid_rows, int valid_cols, int lane, const uint16_t * gate = nullptr) {
     const int l32 = lane & 31;
@@ -684,16 +767,18 @@ TGO_DEVICE void store_rows_32x128(uint16_t * stage, const V16 (&tiles)[4], uint1
     if (!WIDE_ONLY && (row_stride & 7) != 0) {
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
-            const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+            const int across = 8 * (v >> 2) + 4 * half + (v & 3);
+            const int r = TRANSPOSED ? l32 : across;
             if (r < valid_rows) {
 #pragma unroll
                 for (int t = 0; t < 4; ++t) {
-                    if (t * 32 + l32 < valid_cols) {
+                    const int c = t * 32 + (TRANSPOSED ? across : l32);
+                    if (c < valid_cols) {
                         uint16_t value = to_bf16_bits(tiles[t][v]);
                         if (gate != nullptr) {
-                            value = swiglu_bf16(gate[r * row_stride + t * 32 + l32], value);
+                            value = swiglu_bf16(gate[r * row_stride + c], value);
                         }
-                        dst[r * row_stride + t * 32 + l32] = value;
+                        dst[r * row_stride + c] = value;
                     }
                 }
             }
@@ -713,12 +798,24 @@ TGO_DEVICE void store_rows_32x128(uint16_t * stage, const V16 (&tiles)[4], uint1
             }
         }
     }
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+    if constexpr (TRANSPOSED) {
+        static_assert((PITCH / 2) % 4 == 0 && (PITCH / 2) % 64 != 0, "8-byte aligned rows that do not all start in one bank");
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
-            stage[r * PITCH + t * 32 + l32] = to_bf16_bits(tiles[t][v]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                *reinterpret_cast<uint2 *>(&stage[l32 * PITCH + t * 32 + 8 * j + 4 * half]) =
+                    make_uint2(pack_bf16x2(tiles[t][4 * j], tiles[t][4 * j + 1]), pack_bf16x2(tiles[t][4 * j + 2], tiles[t][4 * j + 3]));
+            }
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                stage[r * PITCH + t * 32 + l32] = to_bf16_bits(tiles[t][v]);
+            }
         }
     }
     __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");

@@ -405,37 +405,48 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
                     __builtin_amdgcn_sched_barrier(0);
                 }
             } else {
+                // Two planes: the weight scale is one number per weight row and super-block (the integer sub-scales
+                // are inside the int8 planes), so it is applied once per super-block instead of once per block.  For
+                // that the matrix instructions run with the operands swapped: a lane then holds one activation row
+                // (its eight block scales are eight registers) and 16 weight rows per tile, and per result and block
+                // three vector instructions are left: combine the planes, convert, multiply-add with the
+                // activation scale.
+                float dxb[8];
 #pragma unroll
-            for (int b = 0; b < 8; ++b) {
-                const v4i xfrag = x[b];
-                // scales of the 16 activation rows of this lane's results: wave rows 8j + 4*half + (0..3)
-                float dxv[16];
-#pragma unroll
-                for (int j = 0; j < 4; ++j) {
-                    const float4 d4 =
-                        *reinterpret_cast<const float4 *>(&dxs[buffer][b][wave * 32 + 8 * j + 4 * half]);
-                    dxv[4 * j + 0] = d4.x; dxv[4 * j + 1] = d4.y; dxv[4 * j + 2] = d4.z; dxv[4 * j + 3] = d4.w;
+                for (int b = 0; b < 8; ++b) {
+                    dxb[b] = dxs[buffer][b][wave * 32 + l32];
                 }
 #pragma unroll
                 for (int nt = 0; nt < FWD_NT; ++nt) {
-                    const int slot = ((nt * 8 + b) * 64 + lane) * 16;
-                    const v4i wlo = *reinterpret_cast<const v4i *>(&wq[0][slot]);
-                    const v4i whi = *reinterpret_cast<const v4i *>(&wq[PLANES - 1][slot]);
-                    const float scale = ws[b][nt * 32 + l32];
-                    v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(xfrag, wlo, dot_init, 0, 0, 0);
-                    const v16i dot_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(xfrag, whi, dot_init, 0, 0, 0);
+                    v16f within;
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        dot[v] += dot_hi[v] << 7;
+                    for (int v = 0; v < 16; ++v) within[v] = 0.0f;
+#pragma unroll
+                    for (int b = 0; b < 8; ++b) {
+                        const int slot = ((nt * 8 + b) * 64 + lane) * 16;
+                        const v4i wlo = *reinterpret_cast<const v4i *>(&wq[0][slot]);
+                        const v4i whi = *reinterpret_cast<const v4i *>(&wq[PLANES - 1][slot]);
+                        v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo, x[b], dot_init, 0, 0, 0);
+                        const v16i dot_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi, x[b], dot_init, 0, 0, 0);
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) {
+                            within[v] = fmaf(static_cast<float>(dot[v] + (dot_hi[v] << 7)), dxb[b], within[v]);
+                        }
                     }
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) {
-                        acc[nt][v] = fmaf(static_cast<float>(dot[v]) * scale, dxv[v], acc[nt][v]);
+                    for (int j = 0; j < 4; ++j) {   // weight rows 8j + 4*half + (0..3) of this tile
+                        const float4 d4 = *reinterpret_cast<const float4 *>(&ws[0][nt * 32 + 8 * j + 4 * half]);
+                        acc[nt][4 * j + 0] = fmaf(within[4 * j + 0], d4.x, acc[nt][4 * j + 0]);
+                        acc[nt][4 * j + 1] = fmaf(within[4 * j + 1], d4.y, acc[nt][4 * j + 1]);
+                        acc[nt][4 * j + 2] = fmaf(within[4 * j + 2], d4.z, acc[nt][4 * j + 2]);
+                        acc[nt][4 * j + 3] = fmaf(within[4 * j + 3], d4.w, acc[nt][4 * j + 3]);
                     }
                 }
-                // this block's registers are free: fetch the same block of the next super-block into them
-                load_x(kb * 8 + b + X_AHEAD);
-            }
+                // the super-block is done: fetch the next one's activation fragments
+#pragma unroll
+                for (int b = 0; b < 8; ++b) {
+                    load_x(kb * 8 + b + X_AHEAD);
+                }
             }
         }
     }
@@ -463,14 +474,18 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
 
     // The weight tile is free now: the waves transpose their 32 x 128 results through it (8 KiB each, four
     // waves at a time) so that the output is written in whole 256-byte rows.
-    static_assert(FWD_TN == 128 && sizeof(wq[0]) >= 4 * 32 * 128 * sizeof(uint16_t), "stage fits plane 0");
-    uint16_t * stage = reinterpret_cast<uint16_t *>(&wq[0][0]) + (wave & 3) * (32 * 128);
+    // (the two-plane formats hold transposed results, which need padded rows in the staging area: their weight
+    // tile has a second plane's worth of room)
+    constexpr bool TRANSPOSED = PLANES == 2;
+    constexpr int STAGE_PITCH = TRANSPOSED ? 136 : 128;
+    static_assert(FWD_TN == 128 && sizeof(wq) >= 4 * 32 * STAGE_PITCH * sizeof(uint16_t), "stage fits the weight tile");
+    uint16_t * stage = reinterpret_cast<uint16_t *>(&wq[0][0]) + (wave & 3) * (32 * STAGE_PITCH);
 #pragma unroll
     for (int round = 0; round < S::WAVES / 4; ++round) {
         if ((wave >> 2) == round && wave_active) {
             const int64_t origin = static_cast<int64_t>(wave_row) * a.out_features + n0;
-            store_rows_32x128<128>(stage, acc, y + origin, a.out_features, row_end - wave_row,
-                                   a.out_features - n0, lane, fuse ? a.y + origin : nullptr);
+            store_rows_32x128<STAGE_PITCH, false, TRANSPOSED>(stage, acc, y + origin, a.out_features, row_end - wave_row,
+                                                             a.out_features - n0, lane, fuse ? a.y + origin : nullptr);
         }
         if (round + 1 < S::WAVES / 4) {
             __syncthreads();

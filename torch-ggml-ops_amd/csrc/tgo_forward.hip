@@ -281,7 +281,9 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
         {
             constexpr int UNIT_STEP = THREADS / FWD_TN;
             const uint32_t row = static_cast<uint32_t>(t) & (FWD_TN - 1);
-            const uint32_t first_unit = static_cast<uint32_t>(t) / FWD_TN;
+            // (masked so that the compiler knows the range: unit numbers first_unit + UNIT_STEP * j then split into a
+            // run-time part and constants, and most of the decoders' offset arithmetic folds away)
+            const uint32_t first_unit = (static_cast<uint32_t>(t) / FWD_TN) & (UNIT_STEP - 1);
             const uint8_t * blk = raw + row * SLOT_PITCH + SLOT_FRONT;
             const uint32_t row_slot = ((row >> 5) * 8 * 64 + (row & 31)) * 16;
             if constexpr ((TYPE == Q4_K || TYPE == Q5_K) && UNIT_STEP == 2) {

@@ -26,6 +26,14 @@
  *                   zero block), half-away-from-zero ties, brute force.
  *   mmq_forward   - pinned: equals dequantized-weight x dequantized-activation
  *                   matmul computed independently in numpy float64.
+ *   mmq_forward_half_scales (Q4_K/Q5_K with the four per-block scale values
+ *                   rounded to fp16 where the reference stores them as half2:
+ *                   csrc/vendor/llama_cpp/mmq-load-targets.cuh:190-195,
+ *                   csrc/mmq_core.cuh:202-203, used at
+ *                   mmq-vec-dot-targets.cuh:47-60) - pinned: the rounding helper
+ *                   equals numpy's float16 conversion on every finite half
+ *                   neighbourhood tested (ties, subnormals, overflow), and the
+ *                   function equals a numpy float64 restatement with float16 casts.
  *   linear/grad   - pinned: equal numpy float64 matmuls on the dequantized rows;
  *                   one-hot cotangent reproduces dequantized rows bit for bit.
  */
@@ -70,6 +78,40 @@ static float half_bits_to_float(uint16_t h) {
     float out;
     memcpy(&out, &bits, 4);
     return out;
+}
+
+/* float -> nearest half (ties to even), as bits: overflow to infinity, gradual underflow. */
+static uint16_t float_to_half_bits(float f) {
+    uint32_t bits;
+    memcpy(&bits, &f, 4);
+    const uint16_t sign = (uint16_t)((bits >> 16) & 0x8000u);
+    const uint32_t magnitude = bits & 0x7fffffffu;
+    if (magnitude >= 0x7f800000u) {                       /* infinity or NaN */
+        return (uint16_t)(sign | 0x7c00u | (magnitude > 0x7f800000u ? 0x200u : 0u));
+    }
+    if (magnitude >= 0x477ff000u) {                       /* rounds to 65520 or more: infinity */
+        return (uint16_t)(sign | 0x7c00u);
+    }
+    if (magnitude < 0x38800000u) {                        /* below 2^-14: subnormal half, unit 2^-24 */
+        float absolute;
+        memcpy(&absolute, &magnitude, 4);
+        /* (adding 0.5 * 2^23 units and reading the integer is exact round-to-nearest-even here) */
+        const volatile float shifted = absolute * 16777216.0f + 8388608.0f;
+        const float integer = shifted - 8388608.0f;
+        return (uint16_t)(sign | (uint16_t)integer);
+    }
+    uint32_t rounded = magnitude + 0x0fffu + ((magnitude >> 13) & 1u);   /* nearest even on 13 dropped bits */
+    return (uint16_t)(sign | (uint16_t)((rounded - 0x38000000u) >> 13));
+}
+
+static float round_to_half(float f) {
+    return half_bits_to_float(float_to_half_bits(f));
+}
+
+void tgo_oracle_round_to_half(const float * in, int64_t count, float * out) {
+    for (int64_t i = 0; i < count; ++i) {
+        out[i] = round_to_half(in[i]);
+    }
 }
 
 static float bf16_bits_to_float(uint16_t b) {
@@ -410,6 +452,70 @@ void tgo_oracle_mmq_forward(int qtype, const uint16_t * x, const uint8_t * w,
         }
         free(quant);
         free(scale16);
+        free(min32);
+    }
+    free(qx);
+    free(dx);
+    free(sx);
+}
+
+/* The same algebra for Q4_K / Q5_K with the reference's fp16 storage of the per-block scale values:
+ * weights   (d*sc, -dmin*m) as half2, the product formed in half arithmetic
+ *           (csrc/vendor/llama_cpp/mmq-load-targets.cuh:190-195: dm * make_half2(sc, m));
+ * activation (d, sum) as half2 (csrc/mmq_core.cuh:202-203);
+ * result    sum += dmA.x*dsB.x*dot + dmA.y*dsB.y (mmq-vec-dot-targets.cuh:47-60).
+ * Accumulated in float64: what is modelled is the four roundings to fp16, not the reference's fp32
+ * summation order. */
+void tgo_oracle_mmq_forward_half_scales(int qtype, const uint16_t * x, const uint8_t * w,
+                                        int64_t rows, int64_t n, int64_t k, float * y) {
+    if (qtype != TGO_Q4_K && qtype != TGO_Q5_K) {
+        tgo_oracle_mmq_forward(qtype, x, w, rows, n, k, y);   /* the other formats keep fp32 scales in the reference */
+        return;
+    }
+    const int bytes = tgo_oracle_block_bytes(qtype);
+    const int64_t blocks = k / QK_K;
+    const int64_t groups = k / 32;
+    int8_t * qx = (int8_t *)malloc((size_t)(rows * k));
+    float * dx = (float *)malloc(sizeof(float) * (size_t)(rows * groups));
+    float * sx = (float *)malloc(sizeof(float) * (size_t)(rows * groups));
+    tgo_oracle_quantize_q8_1(x, rows, k, qx, dx, sx);
+    for (int64_t i = 0; i < rows * groups; ++i) {
+        dx[i] = round_to_half(dx[i]);
+        sx[i] = round_to_half(sx[i]);
+    }
+#pragma omp parallel for schedule(static)
+    for (int64_t col = 0; col < n; ++col) {
+        int * quant = (int *)malloc(sizeof(int) * (size_t)k);
+        float * scale32 = (float *)malloc(sizeof(float) * (size_t)groups);
+        float * min32 = (float *)malloc(sizeof(float) * (size_t)groups);
+        for (int64_t b = 0; b < blocks; ++b) {
+            const uint8_t * block = w + (col * blocks + b) * bytes;
+            float d, dmin;
+            block_scales(qtype, block, &d, &dmin);
+            for (int i = 0; i < QK_K; ++i) {
+                const weight_fields f = fields_of(qtype, block, i);
+                quant[b * QK_K + i] = f.quant;
+                if ((i & 31) == 0) {
+                    /* (a product of two halves is exact in fp32, so rounding it is the half multiply) */
+                    scale32[(b * QK_K + i) >> 5] = round_to_half(d * (float)f.sub_scale);
+                    min32[(b * QK_K + i) >> 5] = round_to_half(-dmin * (float)f.sub_min);
+                }
+            }
+        }
+        for (int64_t r = 0; r < rows; ++r) {
+            double acc = 0.0;
+            for (int64_t g = 0; g < groups; ++g) {
+                long dot = 0;
+                for (int i = 0; i < 32; ++i) {
+                    dot += (long)quant[g * 32 + i] * (long)qx[r * k + g * 32 + i];
+                }
+                acc += (double)scale32[g] * (double)dx[r * groups + g] * (double)dot;
+                acc += (double)min32[g] * (double)sx[r * groups + g];
+            }
+            y[r * n + col] = (float)acc;
+        }
+        free(quant);
+        free(scale32);
         free(min32);
     }
     free(qx);

@@ -48,7 +48,9 @@ def lib() -> ctypes.CDLL:
         _lib.tgo_oracle_dequant_bf16.argtypes = [ctypes.c_int, p, i64, i64, p]
         _lib.tgo_oracle_f32_to_bf16.argtypes = [p, i64, p]
         _lib.tgo_oracle_quantize_q8_1.argtypes = [p, i64, i64, p, p, p]
-        for name in ("tgo_oracle_mmq_forward", "tgo_oracle_linear_forward", "tgo_oracle_grad_input"):
+        _lib.tgo_oracle_round_to_half.argtypes = [p, i64, p]
+        for name in ("tgo_oracle_mmq_forward", "tgo_oracle_mmq_forward_half_scales", "tgo_oracle_linear_forward",
+                     "tgo_oracle_grad_input"):
             getattr(_lib, name).argtypes = [ctypes.c_int, p, p, i64, i64, i64, p]
     return _lib
 
@@ -131,6 +133,21 @@ def mmq_forward(qtype, x_bf16, packed, out_features, in_features) -> np.ndarray:
     """Quantized-activation forward algebra, float64 accumulation -> float32 [rows, N]."""
     assert x_bf16.shape[1] == in_features
     return _matmul("tgo_oracle_mmq_forward", qtype, x_bf16, packed, out_features, in_features, out_features)
+
+
+def mmq_forward_half_scales(qtype, x_bf16, packed, out_features, in_features) -> np.ndarray:
+    """mmq_forward with the per-block scale values of Q4_K / Q5_K rounded to fp16 where the reference keeps them
+    as half2 (weights: d*sc and -dmin*m; activations: d and sum); other formats: identical to mmq_forward."""
+    assert x_bf16.shape[1] == in_features
+    return _matmul("tgo_oracle_mmq_forward_half_scales", qtype, x_bf16, packed, out_features, in_features, out_features)
+
+
+def round_to_half(values: np.ndarray) -> np.ndarray:
+    """float32 -> nearest fp16 value (ties to even), returned as float32."""
+    values = _c(values, np.float32)
+    out = np.empty_like(values)
+    lib().tgo_oracle_round_to_half(_ptr(values), values.size, _ptr(out))
+    return out
 
 
 def linear_forward(qtype, x_bf16, packed, out_features, in_features) -> np.ndarray:

@@ -111,6 +111,26 @@ def test_forward_matches_oracle(ops, oracle, qname, shape, n):
         assert max_rel_to_peak(f32(actual).reshape(-1, n), expected) < FORWARD_TOLERANCE
 
 
+@pytest.mark.parametrize("qname", ("Q4_K", "Q5_K"))
+def test_forward_distance_from_the_fp16_scale_numerics(ops, oracle, qname):
+    """For Q4_K / Q5_K the reference stores four per-block scale values as fp16 (weights: d*sc and -dmin*m,
+    csrc/vendor/llama_cpp/mmq-load-targets.cuh:190-195; activations: d and sum, csrc/mmq_core.cuh:202-203); this
+    library keeps them in fp32.  The distance between its output and the oracle's half-scale mode is bounded here:
+    it is the bf16 rounding of the output (up to 2^-9 of an element, 1.1e-3 on norms) plus a few 1e-4 from the fp16 scales."""
+    tgo, _, synth = ops
+    qtype, rows, n, k = QTYPES[qname], 300, 96, 2048
+    host, device = _weight(synth, qtype, n, k, seed=8642 + qtype)
+    x = random_bf16((rows, k), seed=8642)
+    actual = f32(tgo.mmq(x, device, qtype, n))
+    half_mode = oracle.mmq_forward_half_scales(qtype, bits(x), host.numpy(), n, k)
+    fp32_mode = oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k)
+    distance, peak = nrmse(actual, half_mode), max_rel_to_peak(actual, half_mode)
+    between_modes = nrmse(fp32_mode, half_mode)
+    print(f"{qname}: library vs half-scale oracle NRMSE {distance:.2e}, max/peak {peak:.2e}; fp32 vs half-scale oracle {between_modes:.2e}")
+    assert between_modes < 5e-4
+    assert distance < 3e-3 and peak < 5e-3
+
+
 @pytest.mark.parametrize("qname", tuple(QTYPES))
 def test_grad_input_decodes_every_logical_weight_value(ops, oracle, qname):
     _, _, synth = ops

@@ -332,6 +332,83 @@ def test_mmq_forward_equals_dequantized_operands_matmul(oracle, qtype):
     np.testing.assert_allclose(actual, expected, rtol=2e-6, atol=1e-7)
 
 
+def test_round_to_half_is_numpy_float16(oracle):
+    """Every half value, the midpoints between neighbours (ties go to even), values a hair to either side of them,
+    the subnormal range, the overflow threshold 65520 and infinities: same result as numpy's float32 -> float16."""
+    halves = np.arange(0, 0x7C01, dtype=np.uint16).view(np.float16).astype(np.float32)   # 0 .. inf
+    mid = ((halves[:-1].astype(np.float64) + halves[1:].astype(np.float64)) / 2).astype(np.float32)
+    probes = np.concatenate([
+        halves, mid, np.nextafter(mid, np.float32(0)), np.nextafter(mid, np.float32(np.inf)),
+        np.float32([65519.99, 65520.0, 65520.01, 1e6, 3e38, 5.9e-8, 2.9e-8, 3.0e-8, 1e-10, 0.0]),
+    ])
+    probes = np.concatenate([probes, -probes])
+    with np.errstate(over="ignore"):
+        expected = probes.astype(np.float16).astype(np.float32)
+    actual = oracle.round_to_half(probes)
+    np.testing.assert_array_equal(actual.view(np.uint32), expected.view(np.uint32))
+
+
+def _k45_fields(qtype, block):
+    """(quants[256], sc[8], mn[8], d, dmin) of one Q4_K / Q5_K block, read off the layout with numpy."""
+    d = np.frombuffer(bytes(block[0:2]), dtype=np.float16)[0]
+    dmin = np.frombuffer(bytes(block[2:4]), dtype=np.float16)[0]
+    scales = block[4:16].astype(np.int64)
+    sc, mn = np.zeros(8, dtype=np.int64), np.zeros(8, dtype=np.int64)
+    for j in range(8):
+        if j < 4:
+            sc[j], mn[j] = scales[j] & 63, scales[j + 4] & 63
+        else:
+            sc[j] = (scales[j + 4] & 0x0F) | ((scales[j - 4] >> 6) << 4)
+            mn[j] = (scales[j + 4] >> 4) | ((scales[j] >> 6) << 4)
+    low = block[16:144] if qtype == Q4_K else block[48:176]
+    high = None if qtype == Q4_K else block[16:48]
+    quants = np.zeros(256, dtype=np.int64)
+    for chunk in range(4):
+        nibbles = low[32 * chunk: 32 * chunk + 32].astype(np.int64)
+        first, second = nibbles & 0x0F, nibbles >> 4
+        if high is not None:
+            first = first + 16 * ((high.astype(np.int64) >> (2 * chunk)) & 1)
+            second = second + 16 * ((high.astype(np.int64) >> (2 * chunk + 1)) & 1)
+        quants[64 * chunk: 64 * chunk + 32] = first
+        quants[64 * chunk + 32: 64 * chunk + 64] = second
+    return quants, sc, mn, d, dmin
+
+
+@pytest.mark.parametrize("qtype", (Q4_K, Q5_K))
+def test_half_scale_mode_equals_numpy_restatement_and_stays_close_to_fp32_mode(oracle, qtype):
+    """The reference keeps four numbers per 32-value block as fp16 for these two formats: d*sc and -dmin*m of the
+    weights (a half2 product) and d and sum of the activations.  The oracle's half-scale mode is checked against a numpy
+    float64 evaluation with float16 casts in those four places, and its distance from the fp32-scale algebra (what the
+    library computes) is measured: a relative error of at most 2^-11 per factor, far inside the 1e-2 the operator
+    promises."""
+    from torch_ggml_ops import synth
+    from helpers import max_rel_to_peak, nrmse
+
+    rng = np.random.default_rng(900 + qtype)
+    rows, n, k = 6, 9, 1024
+    block_bytes = 144 if qtype == Q4_K else 176
+    packed = synth.random_packed_weight(qtype, (n,), k, seed=70 + qtype).numpy().reshape(n, k // 256, block_bytes)
+    x = _bf16_round(rng.standard_normal((rows, k)).astype(np.float32))
+    q, d, s = oracle.quantize_q8_1(_bf16_bits(x))
+    d16 = d.astype(np.float16).astype(np.float64)
+    s16 = s.astype(np.float16).astype(np.float64)
+    expected = np.zeros((rows, n))
+    for col in range(n):
+        for b in range(k // 256):
+            quants, sc, mn, dw, dmin = _k45_fields(qtype, packed[col, b])
+            scale = (np.float16(dw) * sc.astype(np.float16)).astype(np.float64)       # half multiply
+            minimum = (np.float16(-dmin) * mn.astype(np.float16)).astype(np.float64)
+            for g in range(8):
+                block = 8 * b + g
+                dot = q[:, 32 * block: 32 * block + 32].astype(np.int64) @ quants[32 * g: 32 * g + 32]
+                expected[:, col] += scale[g] * d16[:, block] * dot + minimum[g] * s16[:, block]
+    half_mode = oracle.mmq_forward_half_scales(qtype, _bf16_bits(x), packed, n, k)
+    np.testing.assert_allclose(half_mode, expected, rtol=2e-6, atol=1e-6)
+    fp32_mode = oracle.mmq_forward(qtype, _bf16_bits(x), packed, n, k)
+    assert nrmse(fp32_mode, half_mode) < 1e-3
+    assert max_rel_to_peak(fp32_mode, half_mode) < 1e-3
+
+
 @pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_linear_and_grad_input_equal_float64_matmul(oracle, qtype):
     from torch_ggml_ops import synth

@@ -1571,7 +1571,8 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
         constexpr bool SHORT = decltype(short_tag)::value;
         if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
             const int64_t weight_bytes = static_cast<int64_t>(args.out_features) * args.row_bytes;
-            if (wide_stage_ok(args.packed[0], weight_bytes) &&
+            // (and the rows short enough for the 24-bit multiplies of the unit offsets)
+            if (args.row_bytes < (1 << 24) && wide_stage_ok(args.packed[0], weight_bytes) &&
                 (args.packed[1] == nullptr || wide_stage_ok(args.packed[1], weight_bytes))) {
                 mmq_grad_input_kernel<TYPE, SHORT, true><<<grid, BWD_THREADS, 0, stream>>>(launch_args);
                 return;

@@ -1276,7 +1276,7 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
     }
 }
 
-// ---- short tasks (Q4_K / Q5_K) --------------------------------------------------------------------------------
+// ---- short tasks ----------------------------------------------------------------------------------------------
 // Tasks of at most BACKWARD_SHORT_ROWS rows.  Dequantizing a step's 64 x 128 weights costs the same however few
 // rows multiply them, so here it is nearly all of the work and every wave does it: a wave owns 16 of the step's 64
 // weight rows from the global load to the bf16 tile (packed blocks DEPTH steps ahead in registers, parked in the
@@ -1284,6 +1284,9 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
 // workgroup barrier), one barrier per step publishes the tile, and then every wave multiplies the task's rows with
 // one 32-column slice of it (4 or 8 matrix instructions).  Small footprint: three workgroups share a CU, so one's
 // barrier and memory waits are covered by the others' decoding.  One workgroup per (task, column tile).
+// Q4_K / Q5_K fetch their blocks as the 16-byte units they consist of and have the block-scale stage; the other
+// formats fetch the aligned units that cover their blocks (wide_fetch, callers check wide_stage_ok) and decode
+// 16-value units straight from the parked blocks.
 constexpr int BSH_THREADS = 256;
 constexpr int BSH_ROWS_PER_WAVE = BWD_NS / 4;
 constexpr int BSH_SM_PITCH = BSH_ROWS_PER_WAVE + 1;
@@ -1292,13 +1295,17 @@ constexpr int BSH_DEPTH = 2;
 template <int TYPE>
 __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(const BackwardArgs a) {
     using F = Format<TYPE>;
-    static_assert(TYPE == Q4_K || TYPE == Q5_K, "16-byte aligned blocks only");
-    constexpr int RAW_UNITS = F::BLOCK_BYTES / 16;
+    constexpr bool K45 = TYPE == Q4_K || TYPE == Q5_K;
+    using W = WideStage<TYPE>;
+    constexpr int RAW_UNITS = K45 ? F::BLOCK_BYTES / 16 : W::UNITS;
     constexpr int RAW_REGS = (BSH_ROWS_PER_WAVE * RAW_UNITS + 63) / 64;
+    constexpr int SLOT_PITCH = K45 ? F::RAW_PITCH : W::PITCH;
+    constexpr int SLOT_FRONT = K45 ? 0 : W::FRONT;
     constexpr int QS = TYPE == Q4_K ? 16 : 48;
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t raw_all[4][BSH_ROWS_PER_WAVE * F::RAW_PITCH];
-    __shared__ float2 scale_min_all[4][4 * BSH_SM_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t raw_all[4][BSH_ROWS_PER_WAVE * SLOT_PITCH];
+    __shared__ float2 scale_min_all[K45 ? 4 : 1][4 * BSH_SM_PITCH];
+    __shared__ uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -1325,41 +1332,78 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     const int last = steps - 1;
 
     uint8_t * const raw = raw_all[wave];
-    float2 * const scale_min = scale_min_all[wave];
+    float2 * const scale_min = scale_min_all[K45 ? wave : 0];
+    if constexpr (TYPE == IQ2_S) {
+        expand_iq2s_grid(grid, tid, BSH_THREADS);   // (visible after the barrier that follows the first decode's inputs)
+        __syncthreads();
+    }
 
     // lane offsets of the 16-byte units this lane fetches per step, relative to the step's first weight row
     // (the last step of a source clamps rows past the end of the matrix to its last row)
     const int tail_rows = n_total - (steps_per_source - 1) * BWD_NS;
     uint32_t unit_offset[RAW_REGS], unit_offset_tail[RAW_REGS];
-#pragma unroll
-    for (int i = 0; i < RAW_REGS; ++i) {
-        const int id = min(lane + 64 * i, BSH_ROWS_PER_WAVE * RAW_UNITS - 1);
-        const int row = wave * BSH_ROWS_PER_WAVE + id / RAW_UNITS;
-        const int unit = id % RAW_UNITS;
-        unit_offset[i] = static_cast<uint32_t>(row * a.row_bytes + unit * 16);
-        unit_offset_tail[i] = static_cast<uint32_t>(min(row, tail_rows - 1) * a.row_bytes + unit * 16);
-    }
-    const int64_t expert_offset = static_cast<int64_t>(expert) * a.bytes_per_expert + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
-    auto request = [&](int step, u32x4 (&regs)[RAW_REGS]) __attribute__((always_inline)) {
-        step = min(step, last);
-        const int source = step >= steps_per_source ? 1 : 0;
-        const int n_step = step - source * steps_per_source;
-        const uint8_t * base = (source == 0 ? a.packed[0] : a.packed[1]) + expert_offset +
-                               static_cast<int64_t>(n_step) * BWD_NS * a.row_bytes;
-        const bool tail = n_step == steps_per_source - 1;
-#pragma unroll
-        for (int i = 0; i < RAW_REGS; ++i) {
-            regs[i] = *reinterpret_cast<const u32x4 *>(base + (tail ? unit_offset_tail[i] : unit_offset[i]));
-        }
-    };
-    auto park = [&](const u32x4 (&regs)[RAW_REGS]) __attribute__((always_inline)) {
+    if constexpr (K45) {
 #pragma unroll
         for (int i = 0; i < RAW_REGS; ++i) {
             const int id = min(lane + 64 * i, BSH_ROWS_PER_WAVE * RAW_UNITS - 1);
-            const int row = id / RAW_UNITS;
-            const int unit = id - row * RAW_UNITS;
-            uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
-            dst[0] = regs[i].x; dst[1] = regs[i].y; dst[2] = regs[i].z; dst[3] = regs[i].w;
+            const int row = wave * BSH_ROWS_PER_WAVE + id / RAW_UNITS;
+            const int unit = id % RAW_UNITS;
+            unit_offset[i] = static_cast<uint32_t>(row * a.row_bytes + unit * 16);
+            unit_offset_tail[i] = static_cast<uint32_t>(min(row, tail_rows - 1) * a.row_bytes + unit * 16);
+        }
+    }
+    const int64_t expert_offset = static_cast<int64_t>(expert) * a.bytes_per_expert + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+    // A step's packed blocks in flight: the units themselves (Q4_K / Q5_K) or the covering aligned units.
+    struct InFlight {
+        u32x4 unit[RAW_REGS];
+        WideRegs<K45 ? 1 : RAW_REGS> wide;
+    };
+    // first of this wave's weight rows in a step and how many of them exist (at least one is read: a wave whose rows
+    // all lie past the end of the matrix repeats the last row and decodes zeros)
+    auto wave_rows = [&](int step, const uint8_t *& rows, int & rows_valid, int & n0) __attribute__((always_inline)) {
+        step = min(step, last);
+        const int source = step >= steps_per_source ? 1 : 0;
+        n0 = (step - source * steps_per_source) * BWD_NS;
+        const int first = min(n0 + wave * BSH_ROWS_PER_WAVE, n_total - 1);
+        rows_valid = min(BSH_ROWS_PER_WAVE, n_total - first);
+        rows = (source == 0 ? a.packed[0] : a.packed[1]) + static_cast<int64_t>(expert) * a.bytes_per_expert +
+               static_cast<int64_t>(first) * a.row_bytes;
+    };
+    auto request = [&](int step, InFlight & regs) __attribute__((always_inline)) {
+        if constexpr (K45) {
+            step = min(step, last);
+            const int source = step >= steps_per_source ? 1 : 0;
+            const int n_step = step - source * steps_per_source;
+            const uint8_t * base = (source == 0 ? a.packed[0] : a.packed[1]) + expert_offset +
+                                   static_cast<int64_t>(n_step) * BWD_NS * a.row_bytes;
+            const bool tail = n_step == steps_per_source - 1;
+#pragma unroll
+            for (int i = 0; i < RAW_REGS; ++i) {
+                regs.unit[i] = *reinterpret_cast<const u32x4 *>(base + (tail ? unit_offset_tail[i] : unit_offset[i]));
+            }
+        } else {
+            const uint8_t * rows;
+            int rows_valid, n0;
+            wave_rows(step, rows, rows_valid, n0);
+            wide_fetch<TYPE, BSH_ROWS_PER_WAVE, 64, RAW_REGS>(regs.wide, rows, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
+        }
+    };
+    // (`step`: the one the registers were requested for)
+    auto park = [&](int step, const InFlight & regs) __attribute__((always_inline)) {
+        if constexpr (K45) {
+#pragma unroll
+            for (int i = 0; i < RAW_REGS; ++i) {
+                const int id = min(lane + 64 * i, BSH_ROWS_PER_WAVE * RAW_UNITS - 1);
+                const int row = id / RAW_UNITS;
+                const int unit = id - row * RAW_UNITS;
+                uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
+                dst[0] = regs.unit[i].x; dst[1] = regs.unit[i].y; dst[2] = regs.unit[i].z; dst[3] = regs.unit[i].w;
+            }
+        } else {
+            const uint8_t * rows;
+            int rows_valid, n0;
+            wave_rows(step, rows, rows_valid, n0);
+            wide_park<TYPE, BSH_ROWS_PER_WAVE, 64, RAW_REGS>(raw, regs.wide, rows, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
         }
     };
     auto wave_sync = [&]() __attribute__((always_inline)) {
@@ -1399,7 +1443,34 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     const int position = (word & 7) * 4;
     const int group_local = 2 * (word >> 3) + nibble;
     const int group = 4 * half_block + group_local;
-    auto decode = [&](uint16_t * tile) __attribute__((always_inline)) {
+    auto decode = [&](int step, uint16_t * tile) __attribute__((always_inline)) {
+        if constexpr (!K45) {
+            // 16 rows x 8 units of 16 values: a lane takes one row and two units; neighbouring lanes hold neighbouring
+            // rows of the same values and swap halves so that each writes both rows of one k, four bytes at a time
+            const uint8_t * rows;
+            int rows_valid, n0;
+            wave_rows(step, rows, rows_valid, n0);
+            const int n = lane & 15;
+            uint32_t keep = n0 + wave * BSH_ROWS_PER_WAVE + n < n_total ? 0xffffffffu : 0u;
+            asm volatile("" : "+v"(keep));   // (a mask, not a branch around part of the arithmetic)
+            const uint32_t selector = (lane & 1) != 0 ? 0x03020706u : 0x05040100u;
+#pragma unroll
+            for (int pass = 0; pass < 2; ++pass) {
+                const int unit = (lane >> 4) + 4 * pass;
+                float w[16];
+                decode16_f32<TYPE>(raw + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, w);
+                uint32_t * const pair_row = reinterpret_cast<uint32_t *>(
+                    &tile[(unit * 16 + (lane & 1)) * BWD_PITCH + wave * BSH_ROWS_PER_WAVE + (n & ~1)]);
+#pragma unroll
+                for (int j = 0; j < 16; j += 2) {
+                    const uint32_t own = pack_bf16x2(w[j], w[j + 1]) & keep;
+                    const uint32_t other = static_cast<uint32_t>(
+                        __builtin_amdgcn_mov_dpp(static_cast<int>(own), 0xB1, 0xf, 0xf, true));   // lane ^ 1
+                    pair_row[j * (BWD_PITCH / 2)] = __builtin_amdgcn_perm(other, own, selector);
+                }
+            }
+            return;
+        }
         uint32_t qs[8], qh[8];
         float2 sm[8];
 #pragma unroll
@@ -1476,18 +1547,20 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
         }
     };
 
-    u32x4 ring[BSH_DEPTH][RAW_REGS];
+    InFlight ring[BSH_DEPTH];
 #pragma unroll
     for (int d = 0; d < BSH_DEPTH; ++d) {
         request(d, ring[d]);
     }
     request_cotangent(0);
-    park(ring[0]);
+    park(0, ring[0]);
     request(BSH_DEPTH, ring[0]);
     wave_sync();
-    scales(0);
-    wave_sync();
-    decode(wb[0]);
+    if constexpr (K45) {
+        scales(0);
+        wave_sync();
+    }
+    decode(0, wb[0]);
     __syncthreads();
 #pragma unroll 1
     for (int first = 0; first < steps; first += BSH_DEPTH) {
@@ -1498,16 +1571,18 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
                 const bool more = step + 1 < steps;
                 if (more) {
                     // (this wave's decode of the current step, the last reader of its slot, is behind it in program order)
-                    park(ring[(u + 1) % BSH_DEPTH]);
+                    park(step + 1, ring[(u + 1) % BSH_DEPTH]);
                     request(step + 1 + BSH_DEPTH, ring[(u + 1) % BSH_DEPTH]);
                 }
                 multiply(wb[u & 1]);
                 request_cotangent(step + 1);
                 if (more) {
                     wave_sync();
-                    scales(step + 1);
-                    wave_sync();
-                    decode(wb[(u + 1) & 1]);
+                    if constexpr (K45) {
+                        scales(step + 1);
+                        wave_sync();
+                    }
+                    decode(step + 1, wb[(u + 1) & 1]);
                 }
                 __syncthreads();
             }
@@ -1585,10 +1660,16 @@ static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t s
         BackwardArgs short_args = args;
         short_args.segment = 2;
         bool launched = false;
-        if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
-            // (32-bit lane offsets into the packed cotangent and a step's weight rows, as in the role-split kernel)
-            if (cotangent_workspace_bytes(args.rows, args.out_features) < (int64_t{1} << 32) &&
-                args.row_bytes * 2 * BWD_NS < (int64_t{1} << 32)) {
+        // (32-bit lane offsets into the packed cotangent and a step's weight rows, as in the role-split kernel)
+        if (cotangent_workspace_bytes(args.rows, args.out_features) < (int64_t{1} << 32) &&
+            args.row_bytes * 2 * BWD_NS < (int64_t{1} << 32)) {
+            bool fits = true;
+            if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
+                const int64_t weight_bytes = static_cast<int64_t>(args.out_features) * args.row_bytes;
+                fits = args.row_bytes < (1 << 24) && wide_stage_ok(args.packed[0], weight_bytes) &&
+                       (args.packed[1] == nullptr || wide_stage_ok(args.packed[1], weight_bytes));
+            }
+            if (fits) {
                 mmq_grad_input_short_kernel<TYPE><<<static_cast<unsigned>(total_short), BSH_THREADS, 0, stream>>>(short_args);
                 launched = true;
             }

@@ -169,12 +169,16 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
     if (build.tasks.count != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
         build_tasks(build, threadIdx.x);
     }
-    const int64_t rows_padded = static_cast<int64_t>(gridDim.x) * 32;
+    // Workgroups that are launched together take neighbouring column chunks of the same 32 rows, so that what the
+    // chip reads and writes at any time are whole rows and 8 KiB fragment runs next to each other (with the row
+    // tiles of one chunk launched together instead, the same kernel ran at 4.8 instead of 5.9 TB/s).
+    const int chunks = in_features / 256;
+    const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
     __shared__ __attribute__((aligned(16))) uint8_t tile[8 * 1024];
     __shared__ __attribute__((aligned(16))) float scales[2][8][32];   // d and sum of the tile: [which][block][row]
     const int tid = threadIdx.x;
-    const int row_tile = blockIdx.x;   // 32-row tile
-    const int chunk = blockIdx.y;      // 256-value column chunk
+    const int row_tile = blockIdx.x / chunks;                 // 32-row tile
+    const int chunk = blockIdx.x - row_tile * chunks;         // 256-value column chunk
     const int blocks_per_row = in_features / 32;
     const int lane_k = tid & 31;       // 8 values each
     const int block = lane_k >> 2;     // 32-value block inside the chunk
@@ -247,7 +251,11 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
                                                             gather, input_rows, on_the_side);
         return hipGetLastError();
     }
-    const dim3 grid(static_cast<unsigned>(ws.rows_padded / 32), static_cast<unsigned>(in_features / 256));
+    const int64_t workgroups = ws.rows_padded / 32 * (in_features / 256);
+    if (workgroups > 0x7fffffffLL) {
+        return hipErrorInvalidValue;
+    }
+    const dim3 grid(static_cast<unsigned>(workgroups));
     quantize_q8_1_kernel<<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(rows),
                                                    static_cast<int>(in_features), gather, input_rows, on_the_side);
     return hipGetLastError();

@@ -418,31 +418,57 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
                 for (int b = 0; b < 8; ++b) {
                     dxb[b] = dxs[buffer][b][wave * 32 + l32];
                 }
+                // The 32 (tile, block) steps as a software pipeline, like the single-plane loop: the two fragments of
+                // step t + 2 are read from LDS and the two matrix instructions of step t + 1 issued before the 48
+                // vector instructions of step t, so that neither an LDS round trip nor the matrix latency sits
+                // between a wave's vector instructions.
+                constexpr int STEPS = 8 * FWD_NT;
+                constexpr int RING = 3;   // fragment sets: of the step being read, the one being multiplied and the one being scaled
+                v4i w_lo[RING], w_hi[RING];
+                v16i dot_lo[2], dot_hi[2];
+                v16f within;
+                auto read_step = [&](int step) {
+                    const int nt = step / 8, b = step % 8;
+                    const int slot = ((nt * 8 + b) * 64 + lane) * 16;
+                    w_lo[step % RING] = *reinterpret_cast<const v4i *>(&wq[0][slot]);
+                    w_hi[step % RING] = *reinterpret_cast<const v4i *>(&wq[PLANES - 1][slot]);
+                };
+                auto multiply_step = [&](int step) {
+                    dot_lo[step & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w_lo[step % RING], x[step % 8], dot_init, 0, 0, 0);
+                    dot_hi[step & 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(w_hi[step % RING], x[step % 8], dot_init, 0, 0, 0);
+                };
+                read_step(0);
+                read_step(1);
+                multiply_step(0);
 #pragma unroll
-                for (int nt = 0; nt < FWD_NT; ++nt) {
-                    v16f within;
+                for (int step = 0; step < STEPS; ++step) {
+                    const int nt = step / 8, b = step % 8;
+                    if (step + 2 < STEPS) {
+                        read_step(step + 2);
+                    }
+                    if (step + 1 < STEPS) {
+                        multiply_step(step + 1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if (b == 0) {
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) within[v] = 0.0f;
+                        for (int v = 0; v < 16; ++v) within[v] = 0.0f;
+                    }
 #pragma unroll
-                    for (int b = 0; b < 8; ++b) {
-                        const int slot = ((nt * 8 + b) * 64 + lane) * 16;
-                        const v4i wlo = *reinterpret_cast<const v4i *>(&wq[0][slot]);
-                        const v4i whi = *reinterpret_cast<const v4i *>(&wq[PLANES - 1][slot]);
-                        v16i dot = __builtin_amdgcn_mfma_i32_32x32x32_i8(wlo, x[b], dot_init, 0, 0, 0);
-                        const v16i dot_hi = __builtin_amdgcn_mfma_i32_32x32x32_i8(whi, x[b], dot_init, 0, 0, 0);
+                    for (int v = 0; v < 16; ++v) {
+                        within[v] = fmaf(static_cast<float>(dot_lo[step & 1][v] + (dot_hi[step & 1][v] << 7)), dxb[b], within[v]);
+                    }
+                    if (b == 7) {
 #pragma unroll
-                        for (int v = 0; v < 16; ++v) {
-                            within[v] = fmaf(static_cast<float>(dot[v] + (dot_hi[v] << 7)), dxb[b], within[v]);
+                        for (int j = 0; j < 4; ++j) {   // weight rows 8j + 4*half + (0..3) of this tile
+                            const float4 d4 = *reinterpret_cast<const float4 *>(&ws[0][nt * 32 + 8 * j + 4 * half]);
+                            acc[nt][4 * j + 0] = fmaf(within[4 * j + 0], d4.x, acc[nt][4 * j + 0]);
+                            acc[nt][4 * j + 1] = fmaf(within[4 * j + 1], d4.y, acc[nt][4 * j + 1]);
+                            acc[nt][4 * j + 2] = fmaf(within[4 * j + 2], d4.z, acc[nt][4 * j + 2]);
+                            acc[nt][4 * j + 3] = fmaf(within[4 * j + 3], d4.w, acc[nt][4 * j + 3]);
                         }
                     }
-#pragma unroll
-                    for (int j = 0; j < 4; ++j) {   // weight rows 8j + 4*half + (0..3) of this tile
-                        const float4 d4 = *reinterpret_cast<const float4 *>(&ws[0][nt * 32 + 8 * j + 4 * half]);
-                        acc[nt][4 * j + 0] = fmaf(within[4 * j + 0], d4.x, acc[nt][4 * j + 0]);
-                        acc[nt][4 * j + 1] = fmaf(within[4 * j + 1], d4.y, acc[nt][4 * j + 1]);
-                        acc[nt][4 * j + 2] = fmaf(within[4 * j + 2], d4.z, acc[nt][4 * j + 2]);
-                        acc[nt][4 * j + 3] = fmaf(within[4 * j + 3], d4.w, acc[nt][4 * j + 3]);
-                    }
+                    __builtin_amdgcn_sched_barrier(0);
                 }
                 // the super-block is done: fetch the next one's activation fragments
 #pragma unroll

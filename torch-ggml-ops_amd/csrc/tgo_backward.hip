@@ -28,7 +28,7 @@ namespace tgo {
 
 typedef __bf16 v8bf __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef u32x4_t u32x4;   // (a native vector type: arrays of the uint4 struct end up in scratch memory)
 
 constexpr int BWD_TR = BACKWARD_ROW_TILE;  // rows per workgroup
 constexpr int BWD_TK = 128;                // K columns per workgroup

@@ -42,6 +42,32 @@ EXPERTS = [5, 0, 3, 7, 1, 6, 2, 4]
 
 
 @pytest.mark.parametrize("qname", tuple(QTYPES))
+def test_fused_activation_against_the_oracle(ops, oracle, qname):
+    """Independent of the library's own pair operator: gate and up from the CPU oracle's forward algebra (float64
+    accumulation), the gate rounded to bf16 as the operator stores it, silu(gate) * up in float64.  The fused result
+    may differ from that by the rounding of its own gate (one bf16 ulp of the gate, passed through silu') and its own
+    final rounding, so the comparison is on norms, like the forward's stated tolerance."""
+    from helpers import bits, max_rel_to_peak
+
+    tgo, synth = ops
+    qtype, n, k = QTYPES[qname], 96, 512
+    offsets = np.cumsum(SIZES).tolist()
+    rows = offsets[-1]
+    gate_host = synth.random_packed_weight(qtype, (8, n), k, seed=300 + qtype)
+    up_host = synth.random_packed_weight(qtype, (8, n), k, seed=310 + qtype)
+    x = random_bf16((rows, k), seed=77)
+    metadata = _metadata(EXPERTS, offsets)
+    activated = tgo.grouped_mmq_swiglu(x, gate_host.cuda(), up_host.cuda(), *metadata, qtype, n)
+    gate = oracle.grouped(oracle.mmq_forward, qtype, bits(x), gate_host.numpy(), EXPERTS, offsets, n, k, n)
+    up = oracle.grouped(oracle.mmq_forward, qtype, bits(x), up_host.numpy(), EXPERTS, offsets, n, k, n)
+    gate_bf16 = torch.from_numpy(gate).to(torch.bfloat16).double().numpy()
+    with np.errstate(over="ignore"):   # exp(-gate) of a large negative gate: the quotient is then exactly 0
+        expected = gate_bf16 / (1.0 + np.exp(-gate_bf16)) * up.astype(np.float64)
+    assert nrmse(f32(activated), expected) < 5e-3
+    assert max_rel_to_peak(f32(activated), expected) < 1e-2
+
+
+@pytest.mark.parametrize("qname", tuple(QTYPES))
 @pytest.mark.parametrize("n", (512, 96, 37))
 def test_fused_activation_matches_pair_then_swiglu(ops, qname, n):
     """n = 512: whole tiles; 96: a partial column tile; 37: odd row stride, element-wise stores."""

@@ -594,6 +594,9 @@ def main() -> None:
         help="after the timed region, run one 256 MiB device-to-device copy (a kernel of known traffic for "
         "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters; not timed, not part of the result)",
     )
+    parser.add_argument("--operand", choices=("auto", "half", "int8"), default="auto",
+                        help="matrix operands of the MFMA forward kernels: fp16 numbers holding the exact integers, int8, "
+                        "or the library's default (fp16 for Q6_K and IQ2_S, int8 for the other formats)")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")
@@ -605,6 +608,7 @@ def main() -> None:
 
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    _native.set_forward_operand(args.operand)
     if args.workload == "decode":
         run_decode(args, device)
         return

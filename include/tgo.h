@@ -47,9 +47,10 @@ const char * tgo_last_error(void);
 int tgo_block_bytes(int quant_type);
 
 /* Bytes of the activation workspace the forward entry points need for `rows` rows of
- * `in_features` values: q8_1 blocks (int8 values, one fp32 scale and one fp32 sum per 32 values),
- * rows padded to 32.  The arrangement inside is the library's business (32-row tiles in MFMA
- * fragment order, or plain rows for decode-sized calls); tgo_q8_workspace_unpack reads either.
+ * `in_features` values: q8_1 blocks (two bytes per value, one fp32 scale and one fp32 sum per 32
+ * values), rows padded to 32.  The arrangement inside is the library's business (32-row tiles in MFMA
+ * fragment order holding the quants as fp16 numbers or as int8, see tgo_set_forward_operand, or plain
+ * int8 rows for decode-sized calls); tgo_q8_workspace_unpack reads any of them.
  * Replaces the workspace sizing in csrc/mmq_hip.cu:643-652 and :529-537. */
 int64_t tgo_q8_workspace_bytes(int64_t rows, int64_t in_features);
 
@@ -239,6 +240,20 @@ int tgo_profile_enable(int enabled);
 
 /* Waits for the recorded launches of `kernel` and returns their summed duration and count. */
 int tgo_profile_read(int kernel, double * total_ms, int64_t * launches);
+
+/* Matrix operands of the forward kernels that run on the matrix cores (not the decode-sized GEMV family), a
+ * process-wide setting.  TGO_OPERAND_HALF multiplies fp16 numbers that hold the quantized activations and the
+ * integer weight operands exactly, so the per-block dot products are the same integers as with int8 operands;
+ * TGO_OPERAND_INT8 runs the int8 matrix instruction; TGO_OPERAND_AUTO (default) takes fp16 for the formats whose
+ * integer operand does not fit a byte (Q6_K, IQ2_S) and int8 for the others, and int8 for workspaces that are
+ * quantized before their format is known (tgo_quantize_q8_1 / tgo_mmq_forward_prepared).  The activation workspace
+ * is laid out for one of the two: do not change the setting between quantizing a workspace and using it.
+ * tgo_forward_operand() returns the current setting.  No counterpart in the reference. */
+#define TGO_OPERAND_INT8 0
+#define TGO_OPERAND_HALF 1
+#define TGO_OPERAND_AUTO 2
+int tgo_set_forward_operand(int operand);
+int tgo_forward_operand(void);
 
 #ifdef __cplusplus
 }

@@ -40,8 +40,8 @@ def test_sizes_and_block_bytes(package):
     for qtype, size in synth.BLOCK_BYTES.items():
         assert lib.tgo_block_bytes(qtype) == size
     assert lib.tgo_block_bytes(10) == 0
-    # int8 values + two fp32 per 32 values, rows padded to 32, plus the 1 KiB tail
-    assert lib.tgo_q8_workspace_bytes(33, 512) == 64 * 512 + 2 * 64 * 16 * 4 + 1024
+    # two bytes per value (the quants as fp16 numbers) + two fp32 per 32 values, rows padded to 32, plus the 1 KiB tail
+    assert lib.tgo_q8_workspace_bytes(33, 512) == 2 * 64 * 512 + 2 * 64 * 16 * 4 + 1024
     assert lib.tgo_q8_workspace_bytes(0, 512) == 0
     assert lib.tgo_task_workspace_bytes(100, 7) % 16 == 0
     assert lib.tgo_task_workspace_bytes(100, 7) >= 4 * (1 + 3 * (13 + 7))

@@ -1,0 +1,179 @@
+"""The forward kernels under both kinds of matrix operand (run with -m gpu).
+
+The library multiplies either int8 values or fp16 numbers that hold the same integers exactly
+(`tgo_set_forward_operand`); by default the format decides.  Every check here runs once with each kind
+forced, for all five formats: the quantizer's workspace against the oracle bit for bit, dense, grouped,
+pair and fused-SwiGLU results against the oracle's forward algebra, dense == grouped bit for bit, and the
+two kinds against each other (same integers, different order of the fp32 scale products).
+"""
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import QTYPES, assert_matches_f32_reference, bits, f32, max_rel_to_peak, nrmse, random_bf16
+
+pytestmark = pytest.mark.gpu
+
+FORWARD_TOLERANCE = 1e-2   # against dequantize-then-matmul, as in the dense tests
+
+
+@pytest.fixture(scope="module")
+def ops():
+    import torch_ggml_ops
+    from torch_ggml_ops import _native, synth
+
+    assert torch.cuda.is_available()
+    return torch_ggml_ops, _native, synth
+
+
+@pytest.fixture(params=("int8", "half"))
+def operand(request, ops):
+    _, native, _ = ops
+    native.set_forward_operand(request.param)
+    assert native.forward_operand() == request.param
+    yield request.param
+    native.set_forward_operand("auto")
+
+
+def _metadata(experts, offsets):
+    return (
+        torch.tensor(experts, device="cuda", dtype=torch.int64),
+        torch.tensor(offsets, device="cuda", dtype=torch.int32),
+    )
+
+
+def test_setting_is_validated_and_defaults_to_auto(ops):
+    _, native, _ = ops
+    assert native.forward_operand() == "auto"
+    assert native.lib.tgo_set_forward_operand(7) != 0
+    assert "operand" in native.lib.tgo_last_error().decode()
+    assert native.forward_operand() == "auto"
+
+
+@pytest.mark.parametrize("rows,k", [(33, 512), (129, 2048)])
+def test_workspace_holds_the_oracle_quants(ops, oracle, operand, rows, k):
+    """The format-less quantizer entry follows a forced setting; its fp16 tiles unpack to the same int8 values."""
+    _, native, _ = ops
+    x = random_bf16((rows, k), seed=70 + rows, scale=2.0)
+    x[0, :32] = 0
+    x[0, 32:64] = torch.tensor([127.0, 0.5, 1.5, 2.5, -0.5, -1.5, -2.5, 63.5, -63.5, 126.5, -126.5, -0.25, 0.25, -0.0, 3.5, -3.5] * 2)
+    workspace = torch.empty(native.lib.tgo_q8_workspace_bytes(rows, k), dtype=torch.uint8, device="cuda")
+    native.check(native.lib.tgo_quantize_q8_1(x.data_ptr(), workspace.data_ptr(), rows, k, None))
+    q = torch.empty(rows, k, dtype=torch.int8, device="cuda")
+    d = torch.empty(rows, k // 32, dtype=torch.float32, device="cuda")
+    s = torch.empty(rows, k // 32, dtype=torch.float32, device="cuda")
+    native.check(native.lib.tgo_q8_workspace_unpack(workspace.data_ptr(), q.data_ptr(), d.data_ptr(), s.data_ptr(), rows, k, None))
+    torch.cuda.synchronize()
+    q_ref, d_ref, s_ref = oracle.quantize_q8_1(bits(x))
+    np.testing.assert_array_equal(q.cpu().numpy(), q_ref)
+    np.testing.assert_array_equal(d.cpu().numpy().view(np.uint32), d_ref.view(np.uint32))
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+
+
+@pytest.mark.parametrize("qname", tuple(QTYPES))
+@pytest.mark.parametrize("rows,n,k", [(33, 37, 2048), (96, 130, 512), (300, 96, 2048), (129, 264, 768), (640, 128, 256)])
+def test_dense_forward_matches_oracle(ops, oracle, operand, qname, rows, n, k):
+    """Row counts around the 32- and 128-row tiles, partial column tiles, odd row strides, K of one to eight
+    super-blocks (768: blocks of the 2-byte aligned formats at every misalignment)."""
+    tgo, _, synth = ops
+    qtype = QTYPES[qname]
+    host = synth.random_packed_weight(qtype, (n,), k, seed=500 + qtype + n)
+    x = random_bf16((rows, k), seed=rows + k)
+    actual = tgo.mmq(x, host.cuda(), qtype, n)
+    assert torch.isfinite(actual).all()
+    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k))
+    expected = oracle.linear_forward(qtype, bits(x), host.numpy(), n, k)
+    assert nrmse(f32(actual), expected) < FORWARD_TOLERANCE
+    assert max_rel_to_peak(f32(actual), expected) < FORWARD_TOLERANCE
+
+
+@pytest.mark.parametrize("qname", tuple(QTYPES))
+def test_extreme_blocks_stay_exact(ops, oracle, operand, qname):
+    """All-ones block bytes (largest quants and sub-scales) against activations of +-amax only: the integer dot
+    products reach their largest magnitudes, which the fp16 operands must still hold exactly."""
+    tgo, native, _ = ops
+    qtype, rows, n, k = QTYPES[qname], 64, 64, 512
+    block = native.lib.tgo_block_bytes(qtype)
+    rng = np.random.default_rng(qtype)
+    raw = np.full((n, k // 256, block), 0xFF, dtype=np.uint8)
+    raw[n // 2 :] = rng.choice(np.array([0x00, 0xFF, 0x80, 0x7F], dtype=np.uint8), size=raw[n // 2 :].shape)
+    scale_offsets = {11: (108,), 12: (0, 2), 13: (0, 2), 14: (208,), 22: (0,)}[qtype]
+    for offset in scale_offsets:   # fp16 super-block scales: 2^-7, so nothing overflows
+        raw[:, :, offset] = 0x00
+        raw[:, :, offset + 1] = 0x20
+    host = torch.from_numpy(raw.reshape(n, -1))
+    signs = torch.from_numpy(rng.choice(np.array([-1.0, 1.0], dtype=np.float32), size=(rows, k)))
+    x = (signs * 3.0).to(torch.bfloat16).cuda()
+    actual = tgo.mmq(x, host.cuda(), qtype, n)
+    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k))
+
+
+@pytest.mark.parametrize("qname", tuple(QTYPES))
+def test_grouped_forward_matches_oracle_and_dense(ops, oracle, operand, qname):
+    """Groups of 1 to 200 rows (narrow tasks, partial tiles, a group that spans two tiles); every group's slice is
+    also bit-identical to the dense operator on that slice."""
+    tgo, _, synth = ops
+    qtype, n, k = QTYPES[qname], 200, 1024
+    host = synth.random_packed_weight(qtype, (6, n), k, seed=600 + qtype)
+    device = host.cuda()
+    experts, sizes = [5, 0, 2, 3, 1], [1, 33, 200, 31, 97]
+    offsets = np.cumsum(sizes).tolist()
+    x = random_bf16((offsets[-1], k), seed=4321)
+    actual = tgo.grouped_mmq(x, device, *_metadata(experts, offsets), qtype, n)
+    exact = oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n)
+    assert_matches_f32_reference(actual, exact)
+    begin = 0
+    for expert, end in zip(experts, offsets):
+        if end - begin > 32:   # (up to 32 rows a dense call takes the GEMV family, another summation order)
+            dense = tgo.mmq(x[begin:end].clone(), device[expert].clone(), qtype, n)
+            torch.testing.assert_close(actual[begin:end], dense, rtol=0, atol=0)
+        begin = end
+
+
+@pytest.mark.parametrize("qname", tuple(QTYPES))
+def test_pair_and_fused_swiglu(ops, oracle, operand, qname):
+    tgo, _, synth = ops
+    qtype, n, k = QTYPES[qname], 96, 512
+    gate_host = synth.random_packed_weight(qtype, (8, n), k, seed=700 + qtype)
+    up_host = synth.random_packed_weight(qtype, (8, n), k, seed=710 + qtype)
+    experts, sizes = [0, 2, 5, 7], [5, 140, 64, 33]
+    offsets = np.cumsum(sizes).tolist()
+    metadata = _metadata(experts, offsets)
+    x = random_bf16((offsets[-1], k), seed=88)
+    gate, up = tgo.grouped_mmq_pair(x, gate_host.cuda(), up_host.cuda(), *metadata, qtype, n)
+    torch.testing.assert_close(gate, tgo.grouped_mmq(x, gate_host.cuda(), *metadata, qtype, n), rtol=0, atol=0)
+    torch.testing.assert_close(up, tgo.grouped_mmq(x, up_host.cuda(), *metadata, qtype, n), rtol=0, atol=0)
+    gate_ref = oracle.grouped(oracle.mmq_forward, qtype, bits(x), gate_host.numpy(), experts, offsets, n, k, n)
+    up_ref = oracle.grouped(oracle.mmq_forward, qtype, bits(x), up_host.numpy(), experts, offsets, n, k, n)
+    assert_matches_f32_reference(gate, gate_ref)
+    assert_matches_f32_reference(up, up_ref)
+    activated = tgo.grouped_mmq_swiglu(x, gate_host.cuda(), up_host.cuda(), *metadata, qtype, n)
+    gate_bf16 = torch.from_numpy(gate_ref).to(torch.bfloat16).double().numpy()
+    with np.errstate(over="ignore"):
+        expected = gate_bf16 / (1.0 + np.exp(-gate_bf16)) * up_ref.astype(np.float64)
+    assert nrmse(f32(activated), expected) < 5e-3
+    assert max_rel_to_peak(f32(activated), expected) < 1e-2
+
+
+@pytest.mark.parametrize("qname", tuple(QTYPES))
+def test_both_kinds_agree(ops, qname):
+    """Same integer dot products, fp32 scale products in a different order: the results differ by fp32 rounding
+    before the final bf16 rounding, i.e. at most one bf16 ulp here and there."""
+    tgo, native, synth = ops
+    qtype, rows, n, k = QTYPES[qname], 300, 256, 2048
+    weight = synth.random_packed_weight(qtype, (n,), k, seed=800 + qtype).cuda()
+    x = random_bf16((rows, k), seed=55)
+    results = {}
+    try:
+        for kind in ("int8", "half"):
+            native.set_forward_operand(kind)
+            results[kind] = f32(tgo.mmq(x, weight, qtype, n)).astype(np.float64)
+    finally:
+        native.set_forward_operand("auto")
+    difference = np.abs(results["int8"] - results["half"])
+    assert (difference <= np.abs(results["int8"]) * 2.0**-7 + 1e-6 * np.abs(results["int8"]).max()).all()
+    assert nrmse(results["half"], results["int8"]) < 1e-3
+    native.set_forward_operand("auto")
+    chosen = f32(tgo.mmq(x, weight, qtype, n)).astype(np.float64)
+    np.testing.assert_array_equal(chosen, results["half" if qname in ("Q6_K", "IQ2_S") else "int8"])

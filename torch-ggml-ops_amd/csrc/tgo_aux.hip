@@ -61,6 +61,11 @@ hipError_t launch_dequant_bf16(const uint8_t * packed, uint16_t * out, int64_t r
     return hipGetLastError();
 }
 
+// ---- matrix operands of the forward kernels (process-wide) -------------------------------------------
+static int g_forward_operand = OPERAND_AUTO;
+int forward_operand_setting() { return g_forward_operand; }
+void set_forward_operand_setting(int operand) { g_forward_operand = operand; }
+
 // ---- bf16 activations -> q8_1 -------------------------------------------------------------------
 // Arithmetic of the reference quantizer (csrc/mmq_core.cuh:151-209): per 32 values amax, d = amax/127,
 // q = roundf(x * (127/amax)), and the fp32 sum of the values added in the reference's order (four per
@@ -82,7 +87,10 @@ TGO_DEVICE int round_magnitude(float v) {
 // (an arithmetic shift of each half by 15 is the sign mask of the value it holds): (m ^ s) - s with packed 16-bit
 // operations, then one byte permute per four values.
 typedef short short2_t __attribute__((ext_vector_type(2)));
-TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (&packed)[2], float & d, float & total) {
+// `halves`: the same quants as fp16 numbers, two per register (1024 + magnitude is the magnitude placed under the
+// bits of 1024.0; the sign bit is the one of the bf16 value, which sits at the same place of its half-word).
+TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (&packed)[2], float & d, float & total,
+                               uint32_t (&halves)[4]) {
     float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fabsf(x[2]));
     amax = fmaxf(fmaxf(amax, fabsf(x[3])), fabsf(x[4]));
     amax = fmaxf(fmaxf(amax, fabsf(x[5])), fabsf(x[6]));
@@ -108,6 +116,8 @@ TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (
                                                                 round_magnitude(x[2 * pair + 1] * d_inv));
         const short2_t sign = __builtin_bit_cast(short2_t, words[pair]) >> 15;
         signed_pairs[pair] = __builtin_bit_cast(uint32_t, static_cast<short2_t>((magnitudes ^ sign) - sign));
+        halves[pair] = half2_add(__builtin_bit_cast(uint32_t, magnitudes) | 0x64006400u, half2_of(-1024)) |
+                       (words[pair] & 0x80008000u);
     }
     // low byte of each 16-bit half: bytes 0 and 2 of the first word, then of the second
     packed[0] = __builtin_amdgcn_perm(signed_pairs[1], signed_pairs[0], 0x06040200u);
@@ -148,9 +158,9 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
     }
     float x[8];
     unpack_bf16x8(bits, x);
-    uint32_t packed[2];
+    uint32_t packed[2], halves[4];
     float d, total;
-    quantize_eight(bits, x, packed, d, total);
+    quantize_eight(bits, x, packed, d, total, halves);
     *reinterpret_cast<uint2 *>(q_out + static_cast<int64_t>(row) * in_features + k) = make_uint2(packed[0], packed[1]);
     if ((threadIdx.x & 3) == 0) {
         const int64_t block = static_cast<int64_t>(row) * (in_features / 32) + k / 32;
@@ -159,6 +169,9 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
     }
 }
 
+// HALF: the quants leave as fp16 numbers for the fp16-operand forward kernels, 16 KiB per workgroup: per 32-value
+// block two 1 KiB slabs (k-halves of 16 values), each 64 pieces of eight values = (eighth of the k-half, row).
+template <bool HALF>
 __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __restrict__ input,
                                                            int8_t * __restrict__ q_out,
                                                            float * __restrict__ d_out,
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
     // tiles of one chunk launched together instead, the same kernel ran at 4.8 instead of 5.9 TB/s).
     const int chunks = in_features / 256;
     const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
-    __shared__ __attribute__((aligned(16))) uint8_t tile[8 * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[(HALF ? 16 : 8) * 1024];
     __shared__ __attribute__((aligned(16))) float scales[2][8][32];   // d and sum of the tile: [which][block][row]
     const int tid = threadIdx.x;
     const int row_tile = blockIdx.x / chunks;                 // 32-row tile
@@ -214,12 +227,18 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
         float x[8];
         const uint4 row_bits = present[pass] ? bits[pass] : uint4{0, 0, 0, 0};
         unpack_bf16x8(row_bits, x);
-        uint32_t packed[2];
+        uint32_t packed[2], halves[4];
         float d, total;
-        quantize_eight(row_bits, x, packed, d, total);
+        quantize_eight(row_bits, x, packed, d, total, halves);
         const int half = quarter >> 1;
-        uint2 * dst = reinterpret_cast<uint2 *>(tile + block * 1024 + (rr + 32 * half) * 16 + 8 * (quarter & 1));
-        *dst = make_uint2(packed[0], packed[1]);
+        if constexpr (HALF) {
+            // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
+            *reinterpret_cast<uint4 *>(tile + block * 2048 + half * 1024 + (rr + 32 * (quarter & 1)) * 16) =
+                make_uint4(halves[0], halves[1], halves[2], halves[3]);
+        } else {
+            uint2 * dst = reinterpret_cast<uint2 *>(tile + block * 1024 + (rr + 32 * half) * 16 + 8 * (quarter & 1));
+            *dst = make_uint2(packed[0], packed[1]);
+        }
         if (quarter == 0) {
             scales[0][block][rr] = d;
             scales[1][block][rr] = total;
@@ -233,11 +252,14 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
         *reinterpret_cast<float4 *>(plane + static_cast<int64_t>(chunk * 8 + b) * rows_padded + row_tile * 32 + piece * 4) =
             *reinterpret_cast<const float4 *>(&scales[which][b][piece * 4]);
     }
+    constexpr int BLOCK_BYTES = HALF ? 2048 : 1024;
     uint4 * dst = reinterpret_cast<uint4 *>(
-        q_out + (static_cast<int64_t>(row_tile) * blocks_per_row + chunk * 8) * 1024);
+        q_out + (static_cast<int64_t>(row_tile) * blocks_per_row + chunk * 8) * BLOCK_BYTES);
     const uint4 * src = reinterpret_cast<const uint4 *>(tile);
-    dst[tid] = src[tid];
-    dst[tid + 256] = src[tid + 256];
+#pragma unroll
+    for (int piece = 0; piece < 8 * BLOCK_BYTES / 16 / 256; ++piece) {
+        dst[tid + 256 * piece] = src[tid + 256 * piece];
+    }
 }
 
 hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, int64_t rows,
@@ -256,8 +278,13 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
         return hipErrorInvalidValue;
     }
     const dim3 grid(static_cast<unsigned>(workgroups));
-    quantize_q8_1_kernel<<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(rows),
-                                                   static_cast<int>(in_features), gather, input_rows, on_the_side);
+    if (ws.half_tiles) {
+        quantize_q8_1_kernel<true><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(rows),
+                                                             static_cast<int>(in_features), gather, input_rows, on_the_side);
+    } else {
+        quantize_q8_1_kernel<false><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(rows),
+                                                              static_cast<int>(in_features), gather, input_rows, on_the_side);
+    }
     return hipGetLastError();
 }
 
@@ -266,7 +293,7 @@ __global__ __launch_bounds__(256) void q8_unpack_kernel(const int8_t * __restric
                                                        const float * __restrict__ sum_in,
                                                        int8_t * __restrict__ q, float * __restrict__ d,
                                                        float * __restrict__ sum, int rows,
-                                                       int in_features, bool by_rows) {
+                                                       int in_features, bool by_rows, bool half_tiles) {
     const int64_t index = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     const int64_t total = static_cast<int64_t>(rows) * in_features;
     if (index >= total) {
@@ -284,8 +311,15 @@ __global__ __launch_bounds__(256) void q8_unpack_kernel(const int8_t * __restric
         }
         return;
     }
-    q[index] = q_frag[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 +
-                      ((row & 31) + 32 * half) * 16 + byte];
+    if (half_tiles) {
+        const _Float16 * values = reinterpret_cast<const _Float16 *>(q_frag);
+        q[index] = static_cast<int8_t>(static_cast<float>(
+            values[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 + half * 512 +
+                   ((row & 31) + 32 * (byte >> 3)) * 8 + (byte & 7)]));
+    } else {
+        q[index] = q_frag[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 +
+                          ((row & 31) + 32 * half) * 16 + byte];
+    }
     if ((k & 31) == 0) {
         const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
         d[static_cast<int64_t>(row) * blocks_per_row + block] = d_in[block * rows_padded + row];
@@ -297,7 +331,7 @@ hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float
                             int64_t in_features, hipStream_t stream) {
     const int64_t total = rows * in_features;
     q8_unpack_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(
-        ws.q, ws.d, ws.sum, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features), ws.by_rows);
+        ws.q, ws.d, ws.sum, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features), ws.by_rows, ws.half_tiles);
     return hipGetLastError();
 }
 

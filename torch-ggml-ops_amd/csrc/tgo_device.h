@@ -711,6 +711,137 @@ TGO_DEVICE void decode16_int8(const uint8_t * blk, int u, const uint2 * grid, ui
     }
 }
 
+// ---- exact small integers as fp16 (the forward's matrix operand) --------------------------------
+// The forward multiplies integers: quantized activations (|q| <= 127) and weight operands v = integer sub-scale x
+// quant.  Both are exactly representable in fp16 when |v| <= 2048 (or has enough trailing zero bits), every
+// product is exact in the fp32 accumulator of the matrix instruction, and the sum over a 32-value block stays
+// below 2^24, so the fp16 matrix instruction returns the integer dot product without any rounding, already as
+// a float.  Operand per format:
+//   Q4_K/Q5_K  sc * q            (<= 63 * 31), the weight scale left over is d per super-block
+//   Q3_K       (sc - 32) * q     (|.| <= 128), scale d
+//   IQ2_S      +-(2 s + 1) * m   (<= 31 * 43), scale d / 8
+//   Q6_K       sc * q, |.| <= 4096, as two operands (|sc| & ~15) * q and (|sc| & 15) * q, both with the sign of sc,
+//              whose products accumulate in the same fp32 result (4096 * 127 * 32 < 2^24), scale d
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+
+// Four unsigned bytes -> two registers of two fp16 each holding 1024 + byte: 0x6400 is 1024.0 and its ten
+// mantissa bits count in steps of one, so the byte only has to be placed under the constant.
+TGO_DEVICE void bytes_to_biased_halves(uint32_t bytes, uint32_t & first, uint32_t & second) {
+    first = __builtin_amdgcn_perm(0x64646464u, bytes, 0x04010400u);    // bytes 0, 1
+    second = __builtin_amdgcn_perm(0x64646464u, bytes, 0x04030402u);   // bytes 2, 3
+}
+TGO_DEVICE uint32_t half2_fma(uint32_t a, half2_t b, half2_t c) {
+    return __builtin_bit_cast(uint32_t, __builtin_elementwise_fma(__builtin_bit_cast(half2_t, a), b, c));
+}
+TGO_DEVICE uint32_t half2_add(uint32_t a, half2_t b) {
+    return __builtin_bit_cast(uint32_t, static_cast<half2_t>(__builtin_bit_cast(half2_t, a) + b));
+}
+TGO_DEVICE uint32_t half2_mul(uint32_t a, half2_t b) {
+    return __builtin_bit_cast(uint32_t, static_cast<half2_t>(__builtin_bit_cast(half2_t, a) * b));
+}
+TGO_DEVICE half2_t half2_of(int value) {
+    const _Float16 h = static_cast<_Float16>(static_cast<float>(value));
+    return half2_t{h, h};
+}
+
+// (1024 + byte) pairs times an integer multiplier 0 <= m <= 63, minus the bias: fma(1024 + b, m, -1024 m) is
+// evaluated exactly and b * m is representable.
+struct HalfScale {
+    half2_t multiplier, offset;
+};
+TGO_DEVICE HalfScale half_scale(int multiplier) {
+    return HalfScale{half2_of(multiplier), half2_of(-1024 * multiplier)};
+}
+TGO_DEVICE void scaled_halves(uint32_t bytes, const HalfScale & scale, uint32_t & first, uint32_t & second) {
+    uint32_t a, b;
+    bytes_to_biased_halves(bytes, a, b);
+    first = half2_fma(a, scale.multiplier, scale.offset);
+    second = half2_fma(b, scale.multiplier, scale.offset);
+}
+
+// Values 16u .. 16u+15 of a super-block as the forward's fp16 operand: first[i] holds values 2i and 2i + 1;
+// `second` is Q6_K's low-scale operand (untouched otherwise).  Q4_K/Q5_K have their own loop in the kernel.
+template <int TYPE>
+TGO_DEVICE void decode16_half(const uint8_t * blk, int u, const uint2 * grid, uint32_t (&first)[8], uint32_t (&second)[8]) {
+    static_assert(TYPE == Q3_K || TYPE == Q6_K || TYPE == IQ2_S, "formats with 16-value scale groups");
+    if constexpr (TYPE == Q3_K) {
+        // b = low bits | high bit << 2 in 0..7, quant b - 4, operand (sc - 32) * (b - 4)
+        const int i0 = 16 * u;
+        const uint8_t * qs = blk + 32 + (i0 >> 7) * 32 + (i0 & 31);
+        const uint8_t * hm = blk + (i0 & 31);
+        const int shift_l = 2 * ((i0 & 127) >> 5);
+        const int shift_h = i0 >> 5;
+        const uint8_t * scales = blk + 96;
+        const int low = scales[u & 7] >> (4 * (u >> 3));
+        const int high = scales[8 + (u & 3)] >> (2 * (u >> 2));
+        const int sub = ((low & 0x0f) | ((high & 3) << 4)) - 32;
+        const half2_t multiplier = half2_of(sub);
+        const half2_t unbias = half2_of(-1028);
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t low_bits = lds_u32(qs + 4 * t) >> shift_l;
+            const uint32_t high_bit = lds_u32(hm + 4 * t) >> shift_h;
+            const uint32_t b = (low_bits & 0x03030303u) | ((high_bit & 0x01010101u) << 2);
+            uint32_t p, q;
+            bytes_to_biased_halves(b, p, q);
+            first[2 * t] = half2_mul(half2_add(p, unbias), multiplier);
+            first[2 * t + 1] = half2_mul(half2_add(q, unbias), multiplier);
+        }
+    } else if constexpr (TYPE == Q6_K) {
+        const int chunk = u >> 3;
+        const int rem = (16 * u) & 127;
+        const uint8_t * ql = blk + chunk * 64 + (rem & 63);
+        const uint8_t * qh = blk + 128 + chunk * 32 + ((16 * u) & 31);
+        const int shift_l = 4 * (rem >> 6);
+        const int shift_h = 2 * ((rem >> 5) & 3);
+        const int sc = static_cast<int8_t>(blk[192 + u]);
+        // sign-magnitude split, so that both parts have the sign of sc: the absolute values of all products of a
+        // block then add up to at most 127 * 32 * 32 * 128 < 2^24 and the sum is exact in any order
+        const int magnitude = sc < 0 ? -sc : sc;
+        const int coarse_part = magnitude & ~15, fine_part = magnitude & 15;
+        const half2_t coarse = half2_of(sc < 0 ? -coarse_part : coarse_part);   // multiple of 16: products up to 4096 are exact
+        const half2_t fine = half2_of(sc < 0 ? -fine_part : fine_part);
+        const half2_t unbias = half2_of(-1056);      // 1024 + the quant's offset of 32
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+            const uint32_t low = lds_u32(ql + 4 * t) >> shift_l;
+            const uint32_t high = lds_u32(qh + 4 * t) >> shift_h;
+            const uint32_t b = (low & 0x0f0f0f0fu) | ((high & 0x03030303u) << 4);
+            uint32_t p, q;
+            bytes_to_biased_halves(b, p, q);
+            p = half2_add(p, unbias);
+            q = half2_add(q, unbias);
+            first[2 * t] = half2_mul(p, coarse);
+            first[2 * t + 1] = half2_mul(q, coarse);
+            second[2 * t] = half2_mul(p, fine);
+            second[2 * t + 1] = half2_mul(q, fine);
+        }
+    } else {
+        const uint8_t * qs = blk + 2;
+        const uint32_t idx_pair = lds_u16(qs + 2 * u);
+        const uint32_t sign_pair = lds_u16(qs + 32 + 2 * u);
+        const uint32_t qh = blk[66 + (u >> 1)] >> (4 * (u & 1));
+        const HalfScale scale = half_scale(2 * static_cast<int>((blk[74 + (u >> 1)] >> (4 * (u & 1))) & 0x0f) + 1);
+        // sign of value 2i at bit 2i, of value 2i + 1 at bit 2i + 16: shifted left by 15 - 2i they are the sign
+        // bits of the two halves of register i
+        const uint32_t spread = (sign_pair & 0x5555u) | ((sign_pair & 0xaaaau) << 15);
+#pragma unroll
+        for (int gsel = 0; gsel < 2; ++gsel) {
+            const uint32_t index = ((idx_pair >> (8 * gsel)) & 0xff) | (((qh >> (2 * gsel)) & 3) << 8);
+            const uint2 word = grid[index];
+#pragma unroll
+            for (int part = 0; part < 2; ++part) {
+                uint32_t p, q;
+                scaled_halves(part == 0 ? word.x : word.y, scale, p, q);
+                const int i = 4 * gsel + 2 * part;
+                first[i] = p | ((spread << (15 - 2 * i)) & 0x80008000u);
+                first[i + 1] = q | ((spread << (13 - 2 * i)) & 0x80008000u);
+            }
+        }
+    }
+}
+
 // fp32 scale (and min) of 32-value block b (0..7) of a super-block for the forward algebra.
 template <int TYPE>
 TGO_DEVICE void forward_block_scale(const uint8_t * blk, int b, float & scale, float & minimum) {
@@ -848,14 +979,23 @@ TGO_DEVICE void store_rows_32x128(uint16_t * stage, const V16 (&tiles)[4], uint1
 // The same in two halves for workgroups whose waves each hold one 32x32 tile of a shared 32-row x 128-column
 // block: every wave puts its tile at column `col0` of `stage` (32 x PITCH bf16), and after a barrier
 // store_staged_rows writes the block out with all threads, whole rows at a time.
-template <int PITCH, typename V16>
+// (TRANSPOSED as in store_rows_32x128: the lane holds row l32 and four neighbouring columns per group of four elements)
+template <int PITCH, bool TRANSPOSED = false, typename V16>
 TGO_DEVICE void stage_tile_32x32(uint16_t * stage, const V16 & tile, int col0, int lane) {
     const int l32 = lane & 31;
     const int half = lane >> 5;
+    if constexpr (TRANSPOSED) {
 #pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        const int r = 8 * (v >> 2) + 4 * half + (v & 3);
-        stage[r * PITCH + col0 + l32] = to_bf16_bits(tile[v]);
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<uint2 *>(&stage[l32 * PITCH + col0 + 8 * j + 4 * half]) =
+                make_uint2(pack_bf16x2(tile[4 * j], tile[4 * j + 1]), pack_bf16x2(tile[4 * j + 2], tile[4 * j + 3]));
+        }
+    } else {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int r = 8 * (v >> 2) + 4 * half + (v & 3);
+            stage[r * PITCH + col0 + l32] = to_bf16_bits(tile[v]);
+        }
     }
 }
 

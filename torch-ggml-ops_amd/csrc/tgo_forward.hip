@@ -23,6 +23,7 @@
 #include <type_traits>
 
 #include "tgo_device.h"
+#include "tgo_forward_args.h"
 #include "tgo_launch.h"
 
 namespace tgo {
@@ -30,10 +31,6 @@ namespace tgo {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 typedef float v16f __attribute__((ext_vector_type(16)));
-
-constexpr int FWD_TN = 128;          // weight rows per workgroup
-constexpr int FWD_XCD_RUN = 4;   // consecutive row tasks (mostly tiles of one expert) that share an XCD and its L2
-constexpr int FWD_NT = FWD_TN / 32;  // 32-row weight tiles per wave
 
 // Waves per workgroup; each owns 32 activation rows.  Single-plane formats need about 72 KiB of LDS, so two
 // 4-wave workgroups share a CU; two-plane formats need about 100 KiB and run one 8-wave workgroup per CU.
@@ -44,32 +41,6 @@ struct ForwardShape {
     static constexpr int THREADS = 64 * WAVES;
     static constexpr int ROWS = 32 * WAVES;
     static constexpr int DX_PITCH = ROWS + 4;  // floats per block row of the activation-scale copy
-};
-
-struct ForwardArgs {
-    const uint8_t * packed;
-    const uint8_t * packed_second;   // second projection of a pair, or nullptr
-    int64_t bytes_per_expert;
-    int64_t row_bytes;
-    const int8_t * qx;
-    const float * dx;
-    const float * sx;
-    uint16_t * y;
-    uint16_t * y_second;
-    const int32_t * task_count;   // nullptr: dense
-    const int32_t * task_expert;
-    const int32_t * task_row_start;
-    const int32_t * task_row_end;
-    int rows;
-    int rows_padded;
-    int in_features;
-    int out_features;
-    int n_tiles;
-    int projections;   // 1, or 2 for a pair: both share the task's activations, so their tiles run side by side
-    int swiglu;        // 1: a workgroup runs gate (-> y) then up and stores swiglu(gate, up) -> y_second
-    int task_slots;
-    int dense_row_tile;   // dense calls: rows per workgroup (the format's row tile, or 32 when that fills the chip better)
-    int wide;             // 2-byte aligned formats: the weights may be fetched as aligned 16-byte units (wide_stage_ok)
 };
 
 // LDS of one workgroup.
@@ -522,34 +493,6 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
     }
 }
 
-// The (column tile, projection, task) of this workgroup; false when the slot holds no task.
-template <int TYPE>
-TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second, int & expert, int & row_start,
-                             int & row_end) {
-    using S = ForwardShape<TYPE>;
-    int task;
-    const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + a.dense_row_tile - 1) / a.dense_row_tile;
-    xcd_tile<FWD_XCD_RUN>(blockIdx.x, a.n_tiles * a.projections, tasks, n_tile, task);
-    second = n_tile >= a.n_tiles;
-    n_tile -= second ? a.n_tiles : 0;
-    expert = 0;
-    if (a.task_count != nullptr) {
-        if (task >= tasks) {
-            return false;
-        }
-        expert = a.task_expert[task];
-        row_start = a.task_row_start[task];
-        row_end = a.task_row_end[task];
-    } else {
-        row_start = task * a.dense_row_tile;
-        if (row_start >= a.rows) {
-            return false;
-        }
-        row_end = min(a.rows, row_start + a.dense_row_tile);
-    }
-    return true;
-}
-
 // A task of at most 32 rows has work for one wave only in the usual split (a wave = 32 rows x 128 weight
 // rows).  Such tasks are common under skewed routing, so for them the four waves of a single-plane
 // workgroup take one of the four 32-row weight tiles each instead.  The variants are separate
@@ -581,12 +524,12 @@ __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_ke
     using F = Format<TYPE>;
     using S = ForwardShape<TYPE>;
     constexpr int PLANES = F::PLANES;
-    static_assert(S::ROWS == forward_row_tile(TYPE), "task rows match the workgroup");
+    static_assert(S::ROWS == forward_row_tile(TYPE, false), "task rows match the workgroup");
     __shared__ ForwardLds<TYPE> lds;
 
     int n_tile, expert, row_start, row_end;
     bool second;
-    if (!forward_pick<TYPE>(a, n_tile, second, expert, row_start, row_end)) {
+    if (!forward_pick(a, n_tile, second, expert, row_start, row_end)) {
         return;
     }
     forward_any_task<TYPE>(a, lds, n_tile, second, expert, row_start, row_end);
@@ -604,7 +547,7 @@ __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_sw
 
     int n_tile, expert, row_start, row_end;
     bool second;
-    if (!forward_pick<TYPE>(a, n_tile, second, expert, row_start, row_end)) {
+    if (!forward_pick(a, n_tile, second, expert, row_start, row_end)) {
         return;
     }
 #pragma unroll 1
@@ -666,7 +609,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         args.task_row_start = tasks->row_start;
         args.task_row_end = tasks->row_end;
         args.task_slots = tasks->max_tasks;
-        args.dense_row_tile = forward_row_tile(quant_type);
+        args.dense_row_tile = forward_row_tile(quant_type, ws.half_tiles);
     } else {
         args.task_count = nullptr;
         args.task_expert = nullptr;
@@ -678,7 +621,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         // but their eight waves own 32 rows each: with tiles of 128, 64 or 32 rows only 4, 2 or 1 of them multiply
         // (the others still help to unpack), the vector work of a tile no longer queues two waves deep on every
         // SIMD, and there are 2, 4 or 8 times the workgroups; the largest tile that yields 128 workgroups is taken.
-        int row_tile = forward_row_tile(quant_type);
+        int row_tile = forward_row_tile(quant_type, ws.half_tiles);
         const auto tiles = [&](int tile) { return static_cast<int64_t>(args.n_tiles) * ((rows + tile - 1) / tile); };
         if (row_tile == 128) {
             if (tiles(128) <= 128) {
@@ -691,6 +634,9 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         }
         args.dense_row_tile = row_tile;
         args.task_slots = (rows + row_tile - 1) / row_tile;
+    }
+    if (ws.half_tiles) {
+        return launch_forward_half(args, quant_type, stream);
     }
     switch (quant_type) {
         case Q3_K: return launch_forward_typed<Q3_K>(args, stream);

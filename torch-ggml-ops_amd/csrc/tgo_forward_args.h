@@ -1,0 +1,69 @@
+// What the two forward kernel families (int8 and fp16 matrix operands) share: the launch arguments and the
+// mapping from a workgroup to its (column tile, projection, row task).
+#pragma once
+
+#include "tgo_device.h"
+#include "tgo_launch.h"
+
+namespace tgo {
+
+constexpr int FWD_TN = 128;          // weight rows per workgroup
+constexpr int FWD_XCD_RUN = 4;       // consecutive row tasks (mostly tiles of one expert) that share an XCD and its L2
+constexpr int FWD_NT = FWD_TN / 32;  // 32-row weight tiles per workgroup
+
+struct ForwardArgs {
+    const uint8_t * packed;
+    const uint8_t * packed_second;   // second projection of a pair, or nullptr
+    int64_t bytes_per_expert;
+    int64_t row_bytes;
+    const int8_t * qx;               // int8 tiles, or fp16 tiles (Q8Workspace::half_tiles)
+    const float * dx;
+    const float * sx;
+    uint16_t * y;
+    uint16_t * y_second;
+    const int32_t * task_count;   // nullptr: dense
+    const int32_t * task_expert;
+    const int32_t * task_row_start;
+    const int32_t * task_row_end;
+    int rows;
+    int rows_padded;
+    int in_features;
+    int out_features;
+    int n_tiles;
+    int projections;   // 1, or 2 for a pair: both share the task's activations, so their tiles run side by side
+    int swiglu;        // 1: a workgroup runs gate (-> y) then up and stores swiglu(gate, up) -> y_second
+    int task_slots;
+    int dense_row_tile;   // dense calls: rows per workgroup (the format's row tile, or 32 when that fills the chip better)
+    int wide;             // 2-byte aligned formats: the weights may be fetched as aligned 16-byte units (wide_stage_ok)
+};
+
+// The (column tile, projection, task) of this workgroup; false when the slot holds no task.
+TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second, int & expert, int & row_start,
+                             int & row_end) {
+    int task;
+    const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + a.dense_row_tile - 1) / a.dense_row_tile;
+    xcd_tile<FWD_XCD_RUN>(blockIdx.x, a.n_tiles * a.projections, tasks, n_tile, task);
+    second = n_tile >= a.n_tiles;
+    n_tile -= second ? a.n_tiles : 0;
+    expert = 0;
+    if (a.task_count != nullptr) {
+        if (task >= tasks) {
+            return false;
+        }
+        expert = a.task_expert[task];
+        row_start = a.task_row_start[task];
+        row_end = a.task_row_end[task];
+    } else {
+        row_start = task * a.dense_row_tile;
+        if (row_start >= a.rows) {
+            return false;
+        }
+        row_end = min(a.rows, row_start + a.dense_row_tile);
+    }
+    return true;
+}
+
+// Launch of the fp16-operand kernels for arguments prepared by the common launcher (tgo_forward.hip).
+hipError_t launch_forward_half(const ForwardArgs & args, int quant_type, hipStream_t stream);
+
+}  // namespace tgo

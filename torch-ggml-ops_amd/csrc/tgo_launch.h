@@ -7,9 +7,24 @@
 namespace tgo {
 
 // Row tile of one forward / grad-input task; the task list is built for these.
-// Forward: 256 rows for the formats whose weights unpack into two int8 planes (Q6_K = 14, IQ2_S = 22), 128 rows
-// for the single-plane ones.
-static constexpr int forward_row_tile(int quant_type) { return quant_type == 14 || quant_type == 22 ? 256 : 128; }
+// Forward with int8 operands: 256 rows for the formats whose weights unpack into two int8 planes (Q6_K = 14,
+// IQ2_S = 22), 128 rows for the single-plane ones; with fp16 operands 128 rows for every format.
+static constexpr int forward_row_tile(int quant_type, bool half_operands) {
+    return !half_operands && (quant_type == 14 || quant_type == 22) ? 256 : 128;
+}
+// Matrix operands of the MFMA forward kernels: fp16 numbers holding the exact integers, or int8.  A process-wide
+// setting chooses one of them or (default) lets the format decide: the formats whose integer weight operand does not
+// fit a byte (Q6_K = 14, IQ2_S = 22) run much faster with fp16 operands, the others slightly faster with int8.
+// `quant_type` 0 stands for a workspace that is quantized without knowing the format it will be used with
+// (tgo_quantize_q8_1 / tgo_mmq_forward_prepared): int8 unless fp16 is forced.  The activation workspace is written
+// for one kind of operand, so it must be consumed under the setting it was quantized with.
+enum ForwardOperand : int { OPERAND_INT8 = 0, OPERAND_HALF = 1, OPERAND_AUTO = 2 };
+int forward_operand_setting();
+void set_forward_operand_setting(int operand);
+static inline bool forward_half_operands(int quant_type) {
+    const int setting = forward_operand_setting();
+    return setting == OPERAND_AUTO ? quant_type == 14 || quant_type == 22 : setting == OPERAND_HALF;
+}
 constexpr int BACKWARD_ROW_TILE = 256;
 // Grad-input tasks of at most this many rows (a group's remainder) are listed behind the others and run by a
 // kernel variant whose waves split the K columns of the tile instead of its rows.
@@ -53,33 +68,37 @@ static inline bool use_gemv(int64_t rows, int64_t groups) {
     return groups <= 0 ? rows <= GEMV_DENSE_ROWS : rows <= 4 * groups;
 }
 
-// q8_1 workspace: int8 values, then fp32 scales, then fp32 sums, in one of two layouts over the same bytes.
-// The MFMA kernels want 32-row tiles in fragment order; the GEMV family reads a few rows along K, for which
-// that order would scatter every 16 bytes into a cache line of their own, so calls that take the GEMV family
-// (use_gemv) quantize into plain rows instead.
+// q8_1 workspace: quantized values, then fp32 scales, then fp32 sums, in one of three layouts over the same bytes.
+// The MFMA kernels want 32-row tiles in fragment order, as int8 or (half_tiles) as fp16 numbers holding the same
+// integers; the GEMV family reads a few rows along K, for which that order would scatter every 16 bytes into a
+// cache line of their own, so calls that take the GEMV family (use_gemv) quantize into plain int8 rows instead.
 struct Q8Workspace {
     int8_t * q;     // tiles: [rows_padded/32][K/32][2 halves][32 rows][16 bytes]   by_rows: [rows][K]
+                    // half_tiles: [rows_padded/32][K/32][2 k-halves][2 eighths x 32 rows][8 fp16]
     float * d;      // tiles: [K/32][rows_padded]                                    by_rows: [rows][K/32]
     float * sum;    // same as d
     int64_t rows_padded;
     bool by_rows;
+    bool half_tiles;
 };
 
 static inline int64_t pad_rows(int64_t rows) { return (rows + 31) / 32 * 32; }
 
+// (sized for the fp16 tiles whichever layout a call ends up using)
 static inline int64_t q8_workspace_bytes(int64_t rows, int64_t in_features) {
     const int64_t padded = pad_rows(rows);
     // the 1 KiB tail lets kernels fetch the scales of a whole 32-row tile with 16-byte loads even when the
     // tile starts at the last row
-    return padded * in_features + 2 * padded * (in_features / 32) * static_cast<int64_t>(sizeof(float)) + 1024;
+    return 2 * padded * in_features + 2 * padded * (in_features / 32) * static_cast<int64_t>(sizeof(float)) + 1024;
 }
 
-static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t in_features, bool by_rows) {
+static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t in_features, bool by_rows, int quant_type) {
     Q8Workspace view;
     view.by_rows = by_rows;
+    view.half_tiles = !by_rows && forward_half_operands(quant_type);
     view.rows_padded = pad_rows(rows);
     view.q = static_cast<int8_t *>(base);
-    view.d = reinterpret_cast<float *>(view.q + view.rows_padded * in_features);
+    view.d = reinterpret_cast<float *>(view.q + 2 * view.rows_padded * in_features);
     view.sum = view.d + view.rows_padded * (in_features / 32);
     return view;
 }

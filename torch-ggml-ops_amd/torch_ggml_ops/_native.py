@@ -50,6 +50,8 @@ lib.tgo_grouped_mmq_grad_input.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i64,
 lib.tgo_grouped_mmq_grad_input_weighted.argtypes = [_p, _p, _p, _i64, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
 lib.tgo_profile_enable.argtypes = [_int]
 lib.tgo_profile_read.argtypes = [_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]
+lib.tgo_set_forward_operand.argtypes = [_int]
+lib.tgo_forward_operand.argtypes = []
 
 KERNEL_IDS = {
     "quantize": 0, "build_tasks": 1, "forward": 2, "grad_input": 3, "dequant": 4, "forward_gemv": 5,
@@ -80,7 +82,21 @@ EXPORTS = (
     "tgo_grouped_mmq_grad_input_weighted",
     "tgo_profile_enable",
     "tgo_profile_read",
+    "tgo_set_forward_operand",
+    "tgo_forward_operand",
 )
+
+OPERANDS = {"int8": 0, "half": 1, "auto": 2}
+
+
+def set_forward_operand(operand: str) -> None:
+    """Matrix operands of the MFMA forward kernels: "half" (fp16 numbers holding the exact integers), "int8", or
+    "auto" (the default: fp16 for Q6_K and IQ2_S, int8 otherwise)."""
+    check(lib.tgo_set_forward_operand(OPERANDS[operand]))
+
+
+def forward_operand() -> str:
+    return {value: name for name, value in OPERANDS.items()}[lib.tgo_forward_operand()]
 
 
 def profile_read(kernel: str) -> tuple[float, int]:

@@ -596,7 +596,7 @@ def main() -> None:
     )
     parser.add_argument("--operand", choices=("auto", "half", "int8"), default="auto",
                         help="matrix operands of the MFMA forward kernels: fp16 numbers holding the exact integers, int8, "
-                        "or the library's default (fp16 for Q6_K and IQ2_S, int8 for the other formats)")
+                        "or the library's default (fp16 for IQ2_S, int8 for the other formats)")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this build has no multi-GPU path (run with --gpus 1)")

@@ -244,9 +244,9 @@ int tgo_profile_read(int kernel, double * total_ms, int64_t * launches);
 /* Matrix operands of the forward kernels that run on the matrix cores (not the decode-sized GEMV family), a
  * process-wide setting.  TGO_OPERAND_HALF multiplies fp16 numbers that hold the quantized activations and the
  * integer weight operands exactly, so the per-block dot products are the same integers as with int8 operands;
- * TGO_OPERAND_INT8 runs the int8 matrix instruction; TGO_OPERAND_AUTO (default) takes fp16 for the formats whose
- * integer operand does not fit a byte (Q6_K, IQ2_S) and int8 for the others, and int8 for workspaces that are
- * quantized before their format is known (tgo_quantize_q8_1 / tgo_mmq_forward_prepared).  The activation workspace
+ * TGO_OPERAND_INT8 runs the int8 matrix instruction; TGO_OPERAND_AUTO (default) takes fp16 for IQ2_S (whose integer
+ * operand needs two int8 planes but one fp16 number) and int8 for the other formats, and int8 for workspaces that
+ * are quantized before their format is known (tgo_quantize_q8_1 / tgo_mmq_forward_prepared).  The activation workspace
  * is laid out for one of the two: do not change the setting between quantizing a workspace and using it.
  * tgo_forward_operand() returns the current setting.  No counterpart in the reference. */
 #define TGO_OPERAND_INT8 0

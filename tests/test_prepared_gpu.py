@@ -5,7 +5,7 @@ other tests pin against the CPU oracle): ``mmq_prepared`` must reproduce it bit 
 ``mmq_multi``'s gradient must equal the sum of the projections' ``mmq_grad_input``.
 
 A workspace that is quantized before its weight format is known holds int8 tiles and runs the int8 kernels,
-while ``mmq`` by default multiplies fp16 operands for Q6_K and IQ2_S: bit-for-bit equality therefore holds with the
+while ``mmq`` by default multiplies fp16 operands for IQ2_S: bit-for-bit equality therefore holds with the
 int8 operands forced (and by default for the other formats); under the default the two agree up to fp32 rounding.
 """
 
@@ -36,7 +36,7 @@ def operand(request):
 
 
 def _assert_same(operand, qname, actual, expected):
-    if operand == "int8" or qname not in ("Q6_K", "IQ2_S"):
+    if operand == "int8" or qname != "IQ2_S":
         torch.testing.assert_close(actual, expected, rtol=0, atol=0)
     else:   # one bf16 ulp where the fp32 sums round differently
         torch.testing.assert_close(actual.detach().float(), expected.detach().float(), rtol=2.0**-7,

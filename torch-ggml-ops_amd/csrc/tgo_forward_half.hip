@@ -31,24 +31,32 @@ namespace tgo {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int HALF_THREADS = 256;
-
+// WAVES = 4: 128 activation rows per workgroup, two workgroups per CU; every stage has an unpack phase and a multiply
+// phase with a barrier after each.  WAVES = 8 (half_forward_waves in tgo_launch.h): 256 rows, one workgroup per CU,
+// operand tile, packed blocks and scales double-buffered in LDS; every wave multiplies stage g and then unpacks its
+// share of stage g + 1 before the one barrier of the stage, so the unpack work per activation row halves and a
+// stage costs one barrier instead of two.
 template <int TYPE>
 struct HalfShape {
+    static constexpr int WAVES = half_forward_waves(TYPE);
+    static constexpr bool PIPE = WAVES == 8;
+    static constexpr int THREADS = 64 * WAVES;
     static constexpr int PLANES = TYPE == Q6_K ? 2 : 1;     // fp16 numbers per weight value
     static constexpr int STAGE_BLOCKS = 4 / PLANES;         // 32-value blocks per stage
     static constexpr int STAGES = 8 / STAGE_BLOCKS;
     static constexpr int PLANE_BYTES = FWD_TN * STAGE_BLOCKS * 32 * 2;
+    static constexpr int BUFFERS = PIPE ? 2 : 1;
 };
 
 template <int TYPE>
 struct HalfLds {
     static constexpr int RAW_SLOT = Format<TYPE>::BLOCK_BYTES % 16 == 0 || Format<TYPE>::RAW_PITCH > WideStage<TYPE>::PITCH
                                         ? Format<TYPE>::RAW_PITCH : WideStage<TYPE>::PITCH;
-    alignas(16) uint8_t raw[FWD_TN * RAW_SLOT];                                   // packed blocks of one super-block column
-    alignas(16) uint8_t wq[HalfShape<TYPE>::PLANES][HalfShape<TYPE>::PLANE_BYTES];   // fp16 operand of one stage, fragment order
-    alignas(16) float ws[FWD_TN];                                                 // weight scale of the super-block
-    alignas(16) float wm[Format<TYPE>::HAS_MIN ? 8 : 1][FWD_TN];                  // block minima
+    static constexpr int BUFFERS = HalfShape<TYPE>::BUFFERS;
+    alignas(16) uint8_t raw[BUFFERS][FWD_TN * RAW_SLOT];                                   // packed blocks of a super-block column
+    alignas(16) uint8_t wq[BUFFERS][HalfShape<TYPE>::PLANES][HalfShape<TYPE>::PLANE_BYTES];   // fp16 operand of a stage, fragment order
+    alignas(16) float ws[BUFFERS][FWD_TN];                                                 // weight scale of the super-block
+    alignas(16) float wm[BUFFERS][Format<TYPE>::HAS_MIN ? 8 : 1][FWD_TN];                  // block minima
     uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
 };
 
@@ -75,7 +83,8 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
     constexpr int PLANES = S::PLANES;
     constexpr int SB = S::STAGE_BLOCKS;
     constexpr int STAGES = S::STAGES;
-    constexpr int THREADS = HALF_THREADS;
+    constexpr int THREADS = S::THREADS;
+    constexpr bool PIPE = S::PIPE;
     auto & raw = lds.raw;
     auto & wq = lds.wq;
     auto & ws = lds.ws;
@@ -103,7 +112,7 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
 
     const int granule = NARROW ? 0 : wave;
     const int wave_row = row_start + granule * 32;
-    const bool wave_active = wave_row < row_end;
+    const bool wave_active = wave_row < row_end && (!NARROW || wave < FWD_NT);   // (a narrow task has four tiles)
     int lane_row = wave_row + l32;
     lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
     // Every global address below is a uniform 64-bit base, advanced with scalar arithmetic, plus a 32-bit lane
@@ -146,20 +155,21 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
             wide_fetch<TYPE, FWD_TN, THREADS, WIDE_REGS>(wide_next, tile_weights, static_cast<int>(a.row_bytes), tile_rows, kb, t);
         }
     };
-    auto park_raw = [&](int kb, int t) {
+    auto park_raw = [&](int kb, int t, int buffer) {
+        uint8_t * const raw_slot = &raw[buffer][0];
         if constexpr (RAW_IN_REGS) {
 #pragma unroll
             for (int i = 0; i < RAW_REGS; ++i) {
                 const int id = min(t + THREADS * i, FWD_TN * RAW_UNITS - 1);
                 const int row = static_cast<int>(__umul24(id, UNIT_RECIPROCAL) >> 16);
                 const int unit = id - row * RAW_UNITS;
-                uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
+                uint32_t * dst = reinterpret_cast<uint32_t *>(raw_slot + row * F::RAW_PITCH + unit * 16);
                 dst[0] = raw_next[i].x; dst[1] = raw_next[i].y; dst[2] = raw_next[i].z; dst[3] = raw_next[i].w;
             }
         } else if constexpr (WIDE) {
-            wide_park<TYPE, FWD_TN, THREADS, WIDE_REGS>(raw, wide_next, tile_weights, static_cast<int>(a.row_bytes), tile_rows, kb, t);
+            wide_park<TYPE, FWD_TN, THREADS, WIDE_REGS>(raw_slot, wide_next, tile_weights, static_cast<int>(a.row_bytes), tile_rows, kb, t);
         } else {
-            stage_blocks<TYPE>(raw, weights, a.row_bytes, n0, a.out_features, kb, FWD_TN, t, THREADS);
+            stage_blocks<TYPE>(raw_slot, weights, a.row_bytes, n0, a.out_features, kb, FWD_TN, t, THREADS);
         }
     };
 
@@ -203,15 +213,18 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
     const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 
     // ---- unpack of one stage: raw blocks -> fp16 operand tile -----------------------------------------
-    // A thread keeps its weight row and takes one 16-value half (`fu`) of every 32-value block of the stage, so
-    // consecutive lanes write consecutive 16-byte fragment slots.
-    auto unpack = [&](auto stage_tag, int t) {
+    // A thread keeps its weight row and takes 16-value units of the stage's 32-value blocks, all of the same k-half,
+    // so consecutive lanes write consecutive 16-byte fragment slots.  `share` = t / 128 is wave-uniform.
+    // `source`: buffer of the packed blocks and the scales; `target`: operand tile buffer.
+    constexpr int SHARES = THREADS / FWD_TN;   // 2 or 4 threads per weight row
+    auto unpack = [&](auto stage_tag, int t, int source, int target) {
         constexpr int s = decltype(stage_tag)::value;
         const uint32_t row = static_cast<uint32_t>(t) & (FWD_TN - 1);
-        const uint32_t fu = (static_cast<uint32_t>(t) / FWD_TN) & 1u;   // wave-uniform
-        const uint8_t * blk = raw + row * SLOT_PITCH + SLOT_FRONT;
+        const uint32_t share = (static_cast<uint32_t>(t) / FWD_TN) & (SHARES - 1);
+        const uint32_t fu = share & 1u;   // k-half of the thread's units
+        const uint8_t * blk = &raw[source][0] + row * SLOT_PITCH + SLOT_FRONT;
         // slot of (tile, block b, k-half h, lane = 32 * eighth + row in tile): (((tile * SB + b) * 2 + h) * 64 + lane) * 16
-        uint8_t * const out = &wq[0][0] + (row >> 5) * (SB * 2048) + (row & 31) * 16 + fu * 1024;
+        uint8_t * const out = &wq[target][0][0] + (row >> 5) * (SB * 2048) + (row & 31) * 16 + fu * 1024;
         if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
             constexpr int QS = TYPE == Q4_K ? 16 : 48;
             const uint8_t * half_blk = blk + 16 * fu;
@@ -223,15 +236,22 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
                 }
             }
             const float dmin = half_bits_to_float(lds_u16(blk + 2));
-#pragma unroll
-            for (int p = 0; p < 2; ++p) {
-                // 32 bytes of nibbles: low nibbles are group g, high nibbles group g + 1
-                constexpr int PAIRS = SB / 2;
-                static_assert(PAIRS == 2, "two nibble chunks per stage");
+            // 32 bytes of nibbles: low nibbles are group g, high nibbles group g + 1; a stage has two such chunks,
+            // which a thread takes both (two shares per row) or one of (four shares)
+            static_assert(SB == 4, "two nibble chunks per stage");
+            auto chunk = [&](int p) {
                 const int g = 4 * s + 2 * p;
                 int sc_low, mn_low, sc_high, mn_high;
-                k_scale_min(blk + 4, g, sc_low, mn_low);
-                k_scale_min(blk + 4, g + 1, sc_high, mn_high);
+                if constexpr (s == 0) {   // groups 0..3
+                    sc_low = blk[4 + g] & 0x3f; mn_low = blk[8 + g] & 0x3f;
+                    sc_high = blk[5 + g] & 0x3f; mn_high = blk[9 + g] & 0x3f;
+                } else {                  // groups 4..7
+                    const int j = g - 4;
+                    sc_low = (blk[12 + j] & 0x0f) | ((blk[4 + j] >> 2) & 0x30);
+                    mn_low = (blk[12 + j] >> 4) | ((blk[8 + j] >> 2) & 0x30);
+                    sc_high = (blk[13 + j] & 0x0f) | ((blk[5 + j] >> 2) & 0x30);
+                    mn_high = (blk[13 + j] >> 4) | ((blk[9 + j] >> 2) & 0x30);
+                }
                 const HalfScale scale_low = half_scale(sc_low);
                 const HalfScale scale_high = half_scale(sc_high);
                 uint32_t low[8], high[8];
@@ -242,8 +262,13 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
                     uint32_t bytes_high = (word >> 4) & 0x0f0f0f0fu;
                     if constexpr (TYPE == Q5_K) {
                         // the fifth bit of group g is bit g of the plane byte: moved to bit 4
-                        bytes_low |= (g <= 4 ? planes[w] << (4 - g) : planes[w] >> (g - 4)) & 0x10101010u;
-                        bytes_high |= (g + 1 <= 4 ? planes[w] << (3 - g) : planes[w] >> (g - 3)) & 0x10101010u;
+                        if constexpr (s == 0) {   // g in {0, 2}
+                            bytes_low |= (planes[w] << (4 - g)) & 0x10101010u;
+                            bytes_high |= (planes[w] << (3 - g)) & 0x10101010u;
+                        } else {                  // g in {4, 6}
+                            bytes_low |= (planes[w] >> (g - 4)) & 0x10101010u;
+                            bytes_high |= (planes[w] >> (g - 3)) & 0x10101010u;
+                        }
                     }
                     scaled_halves(bytes_low, scale_low, low[2 * w], low[2 * w + 1]);
                     scaled_halves(bytes_high, scale_high, high[2 * w], high[2 * w + 1]);
@@ -253,18 +278,33 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
                 *reinterpret_cast<uint4 *>(dst + 512) = make_uint4(low[4], low[5], low[6], low[7]);
                 *reinterpret_cast<uint4 *>(dst + 2048) = make_uint4(high[0], high[1], high[2], high[3]);
                 *reinterpret_cast<uint4 *>(dst + 2048 + 512) = make_uint4(high[4], high[5], high[6], high[7]);
-                if (fu == static_cast<uint32_t>(p)) {   // uniform: each half of the workgroup writes two of the four minima
-                    wm[g][row] = dmin * static_cast<float>(mn_low);
-                    wm[g + 1][row] = dmin * static_cast<float>(mn_high);
+                return make_float2(dmin * static_cast<float>(mn_low), dmin * static_cast<float>(mn_high));
+            };
+            if constexpr (SHARES == 4) {
+                const int p = static_cast<int>(share >> 1);
+                const float2 minima = chunk(p);
+                if (fu == 0) {   // uniform
+                    wm[source][4 * s + 2 * p][row] = minima.x;
+                    wm[source][4 * s + 2 * p + 1][row] = minima.y;
+                }
+            } else {
+#pragma unroll
+                for (int p = 0; p < 2; ++p) {
+                    const float2 minima = chunk(p);
+                    if (fu == static_cast<uint32_t>(p)) {   // uniform: each half of the workgroup writes two of the four minima
+                        wm[source][4 * s + 2 * p][row] = minima.x;
+                        wm[source][4 * s + 2 * p + 1][row] = minima.y;
+                    }
                 }
             }
         } else {
 #pragma unroll
-            for (int j = 0; j < SB; ++j) {
-                const uint32_t unit = 2 * (SB * s + j) + fu;
+            for (int j = 0; j < 2 * SB / SHARES; ++j) {
+                const uint32_t local = share + SHARES * j;         // unit within the stage: block local / 2, k-half local % 2
+                const uint32_t unit = 2 * SB * s + local;
                 uint32_t first[8], second_plane[8];
                 decode16_half<TYPE>(blk, unit, grid, first, second_plane);
-                uint8_t * dst = out + j * 2048;
+                uint8_t * dst = out + (local >> 1) * 2048;
                 *reinterpret_cast<uint4 *>(dst) = make_uint4(first[0], first[1], first[2], first[3]);
                 *reinterpret_cast<uint4 *>(dst + 512) = make_uint4(first[4], first[5], first[6], first[7]);
                 if constexpr (PLANES == 2) {
@@ -274,15 +314,15 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
             }
         }
         if constexpr (s == 0) {
-            if (fu == 0) {
-                ws[row] = half_weight_scale<TYPE>(blk);
+            if (share == 0) {
+                ws[source][row] = half_weight_scale<TYPE>(blk);
             }
         }
     };
 
     // ---- multiply phase of one stage ---------------------------------------------------------------
     auto tile_of = [&](int index) { return NARROW ? wave : index; };
-    auto multiply = [&](auto stage_tag, int kb) {
+    auto multiply = [&](auto stage_tag, int kb, int source, int tile) {   // buffers of the scales and of the operand tile
         constexpr int s = decltype(stage_tag)::value;
         // Software pipeline over the CT x SB (tile, block) steps: the fragments of step t + 2 are read from LDS and
         // the matrix instructions of step t + 1 issued before the 16 vector instructions of step t.
@@ -296,8 +336,8 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
             const int slot = ((nt * SB + b) * 2 * 64 + lane) * 16;
 #pragma unroll
             for (int p = 0; p < PLANES; ++p) {
-                w[t % RING][p][0] = *reinterpret_cast<const half8_t *>(&wq[p][slot]);
-                w[t % RING][p][1] = *reinterpret_cast<const half8_t *>(&wq[p][slot + 1024]);
+                w[t % RING][p][0] = *reinterpret_cast<const half8_t *>(&wq[tile][p][slot]);
+                w[t % RING][p][1] = *reinterpret_cast<const half8_t *>(&wq[tile][p][slot + 1024]);
             }
         };
         // The matrix instructions of a step depend on one another (they accumulate into the same result), and a wave
@@ -339,6 +379,10 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
                 for (int v = part * (16 / PARTS); v < (part + 1) * (16 / PARTS); ++v) {
                     within[v] = b == 0 ? dot[t & 1][v] * dxb[0] : __builtin_fmaf(dot[t & 1][v], dxb[b], within[v]);
                 }
+                // (the vector instructions above have no ordering of their own against the scheduling barriers, and
+                // instruction selection may otherwise place them a whole phase later, with every matrix result kept
+                // alive until then: an empty statement that "uses" them holds them here)
+                asm volatile("" : "+v"(within));
                 if (part + 1 < PARTS) {
                     __builtin_amdgcn_sched_barrier(0);
                 }
@@ -347,12 +391,13 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
                 // the tile's share of the stage is complete: apply the weight scales (weight rows 8j + 4*half + 0..3)
 #pragma unroll
                 for (int j = 0; j < 4; ++j) {
-                    const float4 d4 = *reinterpret_cast<const float4 *>(&ws[tile_of(nt) * 32 + 8 * j + 4 * half]);
+                    const float4 d4 = *reinterpret_cast<const float4 *>(&ws[source][tile_of(nt) * 32 + 8 * j + 4 * half]);
                     acc[nt][4 * j + 0] = __builtin_fmaf(within[4 * j + 0], d4.x, acc[nt][4 * j + 0]);
                     acc[nt][4 * j + 1] = __builtin_fmaf(within[4 * j + 1], d4.y, acc[nt][4 * j + 1]);
                     acc[nt][4 * j + 2] = __builtin_fmaf(within[4 * j + 2], d4.z, acc[nt][4 * j + 2]);
                     acc[nt][4 * j + 3] = __builtin_fmaf(within[4 * j + 3], d4.w, acc[nt][4 * j + 3]);
                 }
+                asm volatile("" : "+v"(acc[nt]));   // (held here like the instructions above)
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -364,48 +409,96 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
 #pragma unroll
                 for (int nt = 0; nt < CT; ++nt) {
                     acc[nt] = __builtin_amdgcn_mfma_f32_32x32x2f32(
-                        wm[s * SB + 2 * j + half][tile_of(nt) * 32 + l32], minus_sum, acc[nt], 0, 0, 0);
+                        wm[source][s * SB + 2 * j + half][tile_of(nt) * 32 + l32], minus_sum, acc[nt], 0, 0, 0);
                 }
             }
         }
         load_stage(kb * 8 + s * SB + SB);   // the following stage (block numbers are clamped)
     };
 
-    // The loop exists once per kind of wave (with rows, without, narrow) instead of branching around the multiply
-    // phase inside one loop: with a branch in the body the compiler's wait-count bookkeeping merges both paths and
-    // ends up waiting for every outstanding load, prefetches included, once per round.
+    // The loop exists once per kind of wave (with rows, without) instead of branching around the multiply phase
+    // inside one loop: with a branch in the body the compiler's wait-count bookkeeping merges both paths and ends up
+    // waiting for every outstanding load, prefetches included, once per round.
     // mode 0: no rows for this wave; 1: multiplies
     auto main_loop = [&](auto mode_tag) {
         constexpr bool ACTIVE = decltype(mode_tag)::value != 0;
+        if constexpr (!PIPE) {
 #pragma unroll 1
-        for (int kb = 0; kb < super_blocks; ++kb) {
-            int t = tid;
-            asm volatile("" : "+v"(t));
-            // (every wave has left the previous round's last unpack phase, the last reader of `raw`)
-            park_raw(kb, t);
-            const int kb_next = kb + 1 < super_blocks ? kb + 1 : kb;   // the last round re-fetches its own blocks
-            auto stage = [&](auto stage_tag) {
-                constexpr int s = decltype(stage_tag)::value;
-                __syncthreads();   // the blocks are parked; nobody still reads the previous stage's operand tile
-                if constexpr (s == STAGES - 1) {
-                    load_raw(kb_next, t);
+            for (int kb = 0; kb < super_blocks; ++kb) {
+                int t = tid;
+                asm volatile("" : "+v"(t));
+                // (every wave has left the previous round's last unpack phase, the last reader of `raw`)
+                park_raw(kb, t, 0);
+                const int kb_next = kb + 1 < super_blocks ? kb + 1 : kb;   // the last round re-fetches its own blocks
+                auto stage = [&](auto stage_tag) {
+                    constexpr int s = decltype(stage_tag)::value;
+                    __syncthreads();   // the blocks are parked; nobody still reads the previous stage's operand tile
+                    if constexpr (s == STAGES - 1) {
+                        load_raw(kb_next, t);
+                    }
+                    unpack(stage_tag, t, 0, 0);
+                    __syncthreads();
+                    if constexpr (ACTIVE) {
+                        multiply(stage_tag, kb, 0, 0);
+                    }
+                };
+                stage(std::integral_constant<int, 0>{});
+                stage(std::integral_constant<int, 1>{});
+                if constexpr (STAGES == 4) {
+                    stage(std::integral_constant<int, 2>{});
+                    stage(std::integral_constant<int, 3>{});
                 }
-                unpack(stage_tag, t);
+            }
+        } else {
+            // Stage g is multiplied from operand tile g % 2 while stage g + 1 is unpacked into the other one; the
+            // packed blocks of super-block kb + 1 are requested at the start of kb's last stage but one, parked at
+            // its end in raw[(kb + 1) % 2], and first read one barrier later, by the unpack of (kb + 1, stage 0)
+            // during kb's last stage.  Scales and minima follow the super-block's parity like the packed blocks.
+            {
+                int t = tid;
+                asm volatile("" : "+v"(t));
+                park_raw(0, t, 0);
                 __syncthreads();
-                if constexpr (ACTIVE) {
-                    multiply(stage_tag, kb);
+                unpack(std::integral_constant<int, 0>{}, t, 0, 0);
+                __syncthreads();
+            }
+#pragma unroll 1
+            for (int kb = 0; kb < super_blocks; ++kb) {
+                int t = tid;
+                asm volatile("" : "+v"(t));
+                const int parity = kb & 1;
+                const int kb_next = kb + 1 < super_blocks ? kb + 1 : kb;   // the last round re-fetches its own blocks
+                auto stage = [&](auto stage_tag) {
+                    constexpr int s = decltype(stage_tag)::value;
+                    if constexpr (s == STAGES - 2) {
+                        load_raw(kb_next, t);
+                    }
+                    if constexpr (ACTIVE) {
+                        multiply(stage_tag, kb, parity, s & 1);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);   // the phases stay apart: mixed, their registers do not fit
+                    if constexpr (s + 1 < STAGES) {
+                        unpack(std::integral_constant<int, s + 1>{}, t, parity, (s + 1) & 1);
+                    } else {
+                        unpack(std::integral_constant<int, 0>{}, t, parity ^ 1, 0);
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
+                    if constexpr (s == STAGES - 2) {
+                        park_raw(kb_next, t, parity ^ 1);
+                    }
+                    __syncthreads();
+                };
+                stage(std::integral_constant<int, 0>{});
+                stage(std::integral_constant<int, 1>{});
+                if constexpr (STAGES == 4) {
+                    stage(std::integral_constant<int, 2>{});
+                    stage(std::integral_constant<int, 3>{});
                 }
-            };
-            stage(std::integral_constant<int, 0>{});
-            stage(std::integral_constant<int, 1>{});
-            if constexpr (STAGES == 4) {
-                stage(std::integral_constant<int, 2>{});
-                stage(std::integral_constant<int, 3>{});
             }
         }
     };
-    static_assert(STAGES == 2 || STAGES == 4, "stages are written out above");
-    if (NARROW || wave_active) {
+    static_assert((STAGES == 2 || STAGES == 4) && STAGES % 2 == 0, "stages are written out above; operand tiles alternate");
+    if (wave_active) {
         main_loop(std::integral_constant<int, 1>{});
     } else {
         main_loop(std::integral_constant<int, 0>{});
@@ -415,11 +508,13 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
     // The LDS of the packed blocks and the operand tile is free now: the results, which the swapped operands left
     // transposed in the registers, pass through it (rows padded to 136) and leave as whole 256-byte rows.
     constexpr int STAGE_PITCH = 136;
-    static_assert(offsetof(HalfLds<TYPE>, wq) == sizeof(raw), "the operand tile follows the packed blocks");
-    static_assert(sizeof(raw) + sizeof(wq) >= 4 * 32 * STAGE_PITCH * sizeof(uint16_t), "the staging area fits");
-    uint16_t * const stage_base = reinterpret_cast<uint16_t *>(&raw[0]);
+    static_assert(offsetof(HalfLds<TYPE>, wq) == sizeof(raw), "the operand tiles follow the packed blocks");
+    static_assert(sizeof(raw) + sizeof(wq) >= S::WAVES * 32 * STAGE_PITCH * sizeof(uint16_t), "the staging area fits");
+    uint16_t * const stage_base = reinterpret_cast<uint16_t *>(&raw[0][0]);
     if constexpr (NARROW) {
-        stage_tile_32x32<STAGE_PITCH, true>(stage_base, acc[0], wave * 32, lane);
+        if (wave < FWD_NT) {
+            stage_tile_32x32<STAGE_PITCH, true>(stage_base, acc[0], wave * 32, lane);
+        }
         __syncthreads();
         const int64_t origin = static_cast<int64_t>(row_start) * a.out_features + n0;
         store_staged_rows<STAGE_PITCH>(stage_base, y + origin, a.out_features, row_end - row_start, a.out_features - n0, tid,
@@ -456,7 +551,7 @@ TGO_DEVICE void forward_half_any_task(const ForwardArgs & a, HalfLds<TYPE> & lds
 }
 
 template <int TYPE>
-__global__ __launch_bounds__(HALF_THREADS, 2) void mmq_forward_half_kernel(const ForwardArgs a) {
+__global__ __launch_bounds__(HalfShape<TYPE>::THREADS, 2) void mmq_forward_half_kernel(const ForwardArgs a) {
     __shared__ HalfLds<TYPE> lds;
     int n_tile, expert, row_start, row_end;
     bool second;
@@ -471,7 +566,7 @@ __global__ __launch_bounds__(HALF_THREADS, 2) void mmq_forward_half_kernel(const
 // stores and loads of one address stay ordered once the stores have left the wave (the release fence waits for
 // that), and the CU's vector cache is coherent for its own waves.
 template <int TYPE>
-__global__ __launch_bounds__(HALF_THREADS, 2) void mmq_forward_half_swiglu_kernel(const ForwardArgs a) {
+__global__ __launch_bounds__(HalfShape<TYPE>::THREADS, 2) void mmq_forward_half_swiglu_kernel(const ForwardArgs a) {
     __shared__ HalfLds<TYPE> lds;
     int n_tile, expert, row_start, row_end;
     bool second;
@@ -494,9 +589,9 @@ static hipError_t launch_forward_half_typed(const ForwardArgs & args, hipStream_
     }
     const ProfileScope scope(2, stream);
     if (args.swiglu != 0) {
-        mmq_forward_half_swiglu_kernel<TYPE><<<static_cast<unsigned>(total), HALF_THREADS, 0, stream>>>(args);
+        mmq_forward_half_swiglu_kernel<TYPE><<<static_cast<unsigned>(total), HalfShape<TYPE>::THREADS, 0, stream>>>(args);
     } else {
-        mmq_forward_half_kernel<TYPE><<<static_cast<unsigned>(total), HALF_THREADS, 0, stream>>>(args);
+        mmq_forward_half_kernel<TYPE><<<static_cast<unsigned>(total), HalfShape<TYPE>::THREADS, 0, stream>>>(args);
     }
     return hipGetLastError();
 }

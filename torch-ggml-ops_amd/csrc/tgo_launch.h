@@ -8,13 +8,18 @@ namespace tgo {
 
 // Row tile of one forward / grad-input task; the task list is built for these.
 // Forward with int8 operands: 256 rows for the formats whose weights unpack into two int8 planes (Q6_K = 14,
-// IQ2_S = 22), 128 rows for the single-plane ones; with fp16 operands 128 rows for every format.
+// IQ2_S = 22), 128 rows for the single-plane ones; with fp16 operands 32 rows per wave of the format's workgroup.
+// Waves per workgroup of the fp16-operand kernels, 32 activation rows each (8: the pipelined variant, measured 5 to
+// 11 % faster than the 4-wave one for the formats with 16-value scale groups, and no faster for the others).
+static constexpr int half_forward_waves(int quant_type) { return quant_type == 14 || quant_type == 22 ? 8 : 4; }
 static constexpr int forward_row_tile(int quant_type, bool half_operands) {
-    return !half_operands && (quant_type == 14 || quant_type == 22) ? 256 : 128;
+    return half_operands ? 32 * half_forward_waves(quant_type) : (quant_type == 14 || quant_type == 22 ? 256 : 128);
 }
 // Matrix operands of the MFMA forward kernels: fp16 numbers holding the exact integers, or int8.  A process-wide
-// setting chooses one of them or (default) lets the format decide: the formats whose integer weight operand does not
-// fit a byte (Q6_K = 14, IQ2_S = 22) run much faster with fp16 operands, the others slightly faster with int8.
+// setting chooses one of them or (default) lets the format decide: IQ2_S (22), whose integer operand (2 s + 1) * m
+// needs 11 bits and therefore two int8 planes but a single fp16 number, runs a third faster with fp16 operands; the
+// formats whose operand fits a byte run 5 to 10 % faster with int8 (half the operand bytes through LDS and from the
+// workspace), and Q6_K (14) needs two numbers per value either way and runs the same.
 // `quant_type` 0 stands for a workspace that is quantized without knowing the format it will be used with
 // (tgo_quantize_q8_1 / tgo_mmq_forward_prepared): int8 unless fp16 is forced.  The activation workspace is written
 // for one kind of operand, so it must be consumed under the setting it was quantized with.
@@ -23,7 +28,7 @@ int forward_operand_setting();
 void set_forward_operand_setting(int operand);
 static inline bool forward_half_operands(int quant_type) {
     const int setting = forward_operand_setting();
-    return setting == OPERAND_AUTO ? quant_type == 14 || quant_type == 22 : setting == OPERAND_HALF;
+    return setting == OPERAND_AUTO ? quant_type == 22 : setting == OPERAND_HALF;
 }
 constexpr int BACKWARD_ROW_TILE = 256;
 // Grad-input tasks of at most this many rows (a group's remainder) are listed behind the others and run by a

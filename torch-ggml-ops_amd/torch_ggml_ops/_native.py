@@ -91,7 +91,7 @@ OPERANDS = {"int8": 0, "half": 1, "auto": 2}
 
 def set_forward_operand(operand: str) -> None:
     """Matrix operands of the MFMA forward kernels: "half" (fp16 numbers holding the exact integers), "int8", or
-    "auto" (the default: fp16 for Q6_K and IQ2_S, int8 otherwise)."""
+    "auto" (the default: fp16 for IQ2_S, int8 otherwise)."""
     check(lib.tgo_set_forward_operand(OPERANDS[operand]))
 
 

@@ -654,9 +654,12 @@ def main() -> None:
     active = w["indices"].numel()
     weight_bytes = 2 * active * n * (k // 256) * _native.lib.tgo_block_bytes(w["qtype"])
 
+    # the forward multiplies int8 operands, or fp16 numbers holding the same integers (the library's choice for IQ2_S)
+    half_operands = args.operand == "half" or (args.operand == "auto" and args.quant == "IQ2_S")
+    forward_peak = PEAK["bf16"] if half_operands else PEAK["int8"]   # fp16 and bf16 share the dense matrix peak
     # per-launch algorithmic work of each profiled kernel
     per_launch = {
-        "forward": ("mfma", 2 * flops_projection / 1e12, PEAK["int8"], "TFLOP/s"),  # both projections per launch
+        "forward": ("mfma", 2 * flops_projection / 1e12, forward_peak, "TFLOP/s"),  # both projections per launch
         "grad_input": ("mfma", 2 * flops_projection / 1e12, PEAK["bf16"], "TFLOP/s"),  # both products per launch
         "quantize": ("hbm", (rows * k * 2 + rows * k + 2 * rows * (k // 32) * 4) / 1e9, PEAK["hbm"], "GB/s"),
         "pack_cotangent": ("hbm", 2 * 2 * rows * n * 2 / 1e9, PEAK["hbm"], "GB/s"),  # both cotangents read + written
@@ -681,14 +684,14 @@ def main() -> None:
         "traffic": measured_traffic(dominant) if args.quant == "Q5_K" else None,
         "avg_launch_ms": breakdown[dominant]["avg_ms"],
         # achieved / what two fp32 vector operations per matrix-core result allow (forward kernel only)
-        "valu_bound": VALU_BOUND_INT8 if dominant == "forward" else None,
-        "valu_bound_frac": achieved / VALU_BOUND_INT8 if dominant == "forward" else None,
+        "valu_bound": VALU_BOUND_INT8 if dominant == "forward" and not half_operands else None,
+        "valu_bound_frac": achieved / VALU_BOUND_INT8 if dominant == "forward" and not half_operands else None,
     }
     for name in breakdown:
         if name in per_launch:
             b, wk, pk, un = per_launch[name]
             breakdown[name].update({"achieved": wk / (breakdown[name]["avg_ms"] * 1e-3), "unit": un, "frac_of_peak": wk / (breakdown[name]["avg_ms"] * 1e-3) / pk})
-    if "forward" in breakdown:
+    if "forward" in breakdown and not half_operands:
         breakdown["forward"]["valu_bound_frac"] = breakdown["forward"]["achieved"] / VALU_BOUND_INT8
 
     result = {
@@ -702,7 +705,7 @@ def main() -> None:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "int8 (forward dot products) / bf16 (grad-input), fp32 accumulate",
+        "dtype": ("fp16 holding exact integers" if half_operands else "int8") + " (forward dot products) / bf16 (grad-input), fp32 accumulate",
         "data": "synthetic",
         "config": {
             "workload": f"grouped_mmq_pair fwd+bwd: 256 experts, gate+up {args.quant} [512,2048], T=8192 x top-8 "

@@ -89,6 +89,36 @@ def pair_step(w):
     return out_first, out_second, grad_input
 
 
+def measure_pair_format(device, name, qtype, steps=10, warmup=3):
+    """The default workload with another weight format (the reference's model packs its gate and up projections as
+    IQ2_S): step time by the wall clock, kernel times from the event brackets."""
+    from torch_ggml_ops import _native
+
+    w = build_pair_workload(device, qtype=qtype)
+    for _ in range(warmup):
+        pair_step(w)
+    torch.cuda.synchronize()
+    _native.lib.tgo_profile_enable(1)
+    start = time.perf_counter()
+    for _ in range(steps):
+        pair_step(w)
+    torch.cuda.synchronize()
+    elapsed = time.perf_counter() - start
+    kernels = {name_: _native.profile_read(name_) for name_ in ("quantize", "forward", "pack_cotangent", "grad_input")}
+    _native.lib.tgo_profile_enable(0)
+    flops = 4 * 2.0 * w["rows"] * w["n"] * w["k"]
+    record = {
+        "workload": f"grouped_mmq_pair fwd+bwd, gate+up {name} [512,2048], same routing as the headline workload",
+        "value": flops / (elapsed / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": elapsed / steps * 1e3, "steps": steps,
+        "forward_operands": "fp16 numbers holding the exact integers" if _native.forward_operand() == "half" or
+        (_native.forward_operand() == "auto" and qtype == 22) else "int8",
+        "kernels_us": {k: total / launches * 1e3 for k, (total, launches) in kernels.items() if launches},
+    }
+    del w
+    torch.cuda.empty_cache()
+    return record
+
+
 def cpu_baseline_pair(w, budget_seconds=15.0):
     """Dequantize to fp32 with the oracle + torch.matmul, forward and grad-input, group by group."""
     from oracle import gguf_oracle as oracle
@@ -729,6 +759,7 @@ def main() -> None:
             "workload": f"grouped_mmq down projection: 256 experts, Q4_K [2048,512], T=4096 x top-8 ({down['rows']} rows)",
             "forward": down["forward"], "grad_input": down["grad_input"],
         }
+        result["pair_iq2s"] = measure_pair_format(device, "IQ2_S", 22)
         decode = measure_decode(args, device)
         result["decode"] = {
             "workload": "T in {1,4,8} x top-8 over 256 experts: gate+up IQ2_S [512,2048] + down Q6_K [2048,512]; "

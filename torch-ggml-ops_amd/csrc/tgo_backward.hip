@@ -239,7 +239,10 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
     __shared__ __attribute__((aligned(16))) uint8_t raw_odd[WIDE ? BWD_NS * SLOT_PITCH : 16];   // second slot of the WIDE pipeline
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
     __shared__ float2 scale_min[FAST_K45 ? 4 * (BWD_NS + 8) : 1];
-    __shared__ uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
+    // (IQ2_S: the selector table of decode16_bf16; the other formats have no codebook)
+    using Codebook = std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2>;
+    __shared__ Codebook codebook_storage;
+    const Codebook * const grid = &codebook_storage;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -274,7 +277,7 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
         row_end = min(a.rows, row_start + BWD_TR);
     }
     if constexpr (TYPE == IQ2_S) {
-        expand_iq2s_grid(grid, tid, BWD_THREADS);
+        expand_iq2s_selectors(codebook_storage, tid, BWD_THREADS);
     }
 
     const int wave_row = SHORT ? row_start : row_start + wave * 64;
@@ -395,8 +398,8 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                 const int id = tid + BWD_THREADS * pass;
                 const int n = id & 63;
                 const int unit = id >> 6;
-                float w[16];
-                decode16_f32<TYPE>(raw + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, w);
+                uint32_t pairs[8];
+                decode16_bf16<TYPE>(raw + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, pairs);
                 const bool valid = n0 + n < n_total;
                 // Neighbouring lanes hold neighbouring weight rows of the same 16 values of K.  They swap pairs of
                 // bf16 values so that the even lane writes both rows of an even k and the odd lane both rows of the
@@ -405,7 +408,7 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                 uint32_t * const pair_row = reinterpret_cast<uint32_t *>(&tile[(unit * 16 + (lane & 1)) * BWD_PITCH + (n & ~1)]);
 #pragma unroll
                 for (int j = 0; j < 16; j += 2) {
-                    const uint32_t own = valid ? pack_bf16x2(w[j], w[j + 1]) : 0u;
+                    const uint32_t own = valid ? pairs[j / 2] : 0u;
                     const uint32_t other = static_cast<uint32_t>(
                         __builtin_amdgcn_mov_dpp(static_cast<int>(own), 0xB1, 0xf, 0xf, true));   // lane ^ 1
                     pair_row[j * (BWD_PITCH / 2)] = __builtin_amdgcn_perm(other, own, selector);
@@ -539,8 +542,8 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
             const int n0 = (step - source * steps_per_source) * BWD_NS;
             const int n = lane;
             const int unit = wave + 4 * pass;   // (wave-uniform: the unit's shifts and offsets are scalars)
-            float w[16];
-            decode16_f32<TYPE>(slot + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, w);
+            uint32_t pairs[8];
+            decode16_bf16<TYPE>(slot + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, pairs);
             // rows past the end of the weight matrix become zeros (a mask the compiler cannot see through: a visible
             // condition ends up as a branch around part of the arithmetic, which splits the block of code that the
             // matrix and vector instructions are meant to share)
@@ -551,7 +554,7 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
             uint32_t * const pair_row = reinterpret_cast<uint32_t *>(&tile[(unit * 16 + (lane & 1)) * BWD_PITCH + (n & ~1)]);
 #pragma unroll
             for (int j = 0; j < 16; j += 2) {
-                const uint32_t own = pack_bf16x2(w[j], w[j + 1]) & keep;
+                const uint32_t own = pairs[j / 2] & keep;
                 const uint32_t other = static_cast<uint32_t>(
                     __builtin_amdgcn_mov_dpp(static_cast<int>(own), 0xB1, 0xf, 0xf, true));   // lane ^ 1
                 pair_row[j * (BWD_PITCH / 2)] = __builtin_amdgcn_perm(other, own, selector);
@@ -1305,6 +1308,8 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
     __shared__ __attribute__((aligned(16))) uint8_t raw_all[4][BSH_ROWS_PER_WAVE * SLOT_PITCH];
     __shared__ float2 scale_min_all[K45 ? 4 : 1][4 * BSH_SM_PITCH];
+    // (the magnitude grid, not the 16 KiB selector table of decode16_bf16: with that table only two of these
+    // workgroups fit a CU instead of three, which costs more than the cheaper decode brings -- measured)
     __shared__ uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
 
     const int tid = threadIdx.x;
@@ -1457,13 +1462,13 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
 #pragma unroll
             for (int pass = 0; pass < 2; ++pass) {
                 const int unit = (lane >> 4) + 4 * pass;
-                float w[16];
-                decode16_f32<TYPE>(raw + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, w);
+                uint32_t pairs[8];
+                decode16_bf16<TYPE>(raw + n * SLOT_PITCH + SLOT_FRONT, 8 * half_block + unit, grid, pairs);
                 uint32_t * const pair_row = reinterpret_cast<uint32_t *>(
                     &tile[(unit * 16 + (lane & 1)) * BWD_PITCH + wave * BSH_ROWS_PER_WAVE + (n & ~1)]);
 #pragma unroll
                 for (int j = 0; j < 16; j += 2) {
-                    const uint32_t own = pack_bf16x2(w[j], w[j + 1]) & keep;
+                    const uint32_t own = pairs[j / 2] & keep;
                     const uint32_t other = static_cast<uint32_t>(
                         __builtin_amdgcn_mov_dpp(static_cast<int>(own), 0xB1, 0xf, 0xf, true));   // lane ^ 1
                     pair_row[j * (BWD_PITCH / 2)] = __builtin_amdgcn_perm(other, own, selector);

@@ -7,6 +7,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "iq2s_codebook.h"
 #include "tgo_launch.h"
 
@@ -466,6 +468,28 @@ TGO_DEVICE void unpack16(const uint8_t * blk, int u, const uint2 * grid, int (&q
     }
 }
 
+// IQ2_S has only three magnitudes (8, 25, 43), so a 16-value unit, whose values share one fp32 factor t, takes only
+// six different bf16 numbers: +-bf16(t * 8), +-bf16(t * 25), +-bf16(t * 43).  The dequantizing kernels therefore
+// round three products per unit and let every value pick its number with a byte permute instead of converting and
+// multiplying each value: the table below holds, per codebook entry, the permute selectors of its eight values
+// (two values per selector word; a value's two selector bytes are 2 * digit and 2 * digit + 1, which address
+// the pair (bf16(t*8), bf16(t*25)) and, as bytes 4 and 5, bf16(t*43)).  16 KiB of LDS.
+struct Iq2sSelectors {
+    uint4 entry[TGO_IQ2S_GRID_ENTRIES];
+};
+TGO_DEVICE void expand_iq2s_selectors(Iq2sSelectors & table, int tid, int nthreads) {
+    for (int i = tid; i < TGO_IQ2S_GRID_ENTRIES; i += nthreads) {
+        const uint32_t packed = tgo_iq2s_packed[i];
+        uint32_t words[4];
+#pragma unroll
+        for (int p = 0; p < 4; ++p) {
+            const uint32_t first = (packed >> (4 * p)) & 3u, second = (packed >> (4 * p + 2)) & 3u;
+            words[p] = 0x01000100u + first * 0x0202u + second * 0x02020000u;
+        }
+        table.entry[i] = make_uint4(words[0], words[1], words[2], words[3]);
+    }
+}
+
 // fp32 value of 16 consecutive weights, operation order of the reference decoder:
 //   Q4_K/Q5_K (d*sc)*q - dmin*m ; Q3_K/Q6_K (d*sc)*q ; IQ2_S ((d*(0.5+s))*0.25)*q
 template <int TYPE>
@@ -542,6 +566,49 @@ TGO_DEVICE void decode16_f32(const uint8_t * blk, int u, const uint2 * grid, flo
 #pragma unroll
         for (int i = 0; i < 16; ++i) {
             w[i] = scale * static_cast<float>(q[i]);
+        }
+    }
+}
+
+// 16 consecutive weights as bf16, two per word (values 2i and 2i + 1 in word i), bit-identical to rounding
+// decode16_f32's results.  `codebook`: the magnitude grid, or for IQ2_S the selector table above.
+template <int TYPE, typename Codebook>
+TGO_DEVICE void decode16_bf16(const uint8_t * blk, int u, const Codebook * codebook, uint32_t (&pairs)[8]) {
+    if constexpr (TYPE == IQ2_S && std::is_same_v<Codebook, Iq2sSelectors>) {
+        const uint8_t * qs = blk + 2;
+        const uint32_t idx_pair = lds_u16(qs + 2 * u);
+        const uint32_t sign_pair = lds_u16(qs + 32 + 2 * u);
+        const uint32_t qh = blk[66 + (u >> 1)] >> (4 * (u & 1));
+        const int sub = (blk[74 + (u >> 1)] >> (4 * (u & 1))) & 0x0f;
+        // the reference's ((d * (0.5 + s)) * 0.25) * q with q = +-m: the magnitude of the product does not depend on
+        // the signs, and rounding is symmetric, so the three candidates are formed from |t| and every value gets
+        // the sign of t xor its own sign bit
+        const float t = (half_bits_to_float(lds_u16(blk)) * (0.5f + static_cast<float>(sub))) * 0.25f;
+        const float magnitude = __builtin_fabsf(t);
+        const uint32_t low_pair = pack_bf16x2(magnitude * 8.0f, magnitude * 25.0f);
+        const uint32_t high = pack_bf16x2(magnitude * 43.0f, 0.0f);
+        // sign of value 2i at bit 2i, of value 2i + 1 at bit 2i + 16: shifted left by 15 - 2i they are the sign bits of
+        // the two halves of word i
+        uint32_t spread = (sign_pair & 0x5555u) | ((sign_pair & 0xaaaau) << 15);
+        spread ^= static_cast<uint32_t>(static_cast<int>(__builtin_bit_cast(uint32_t, t)) >> 31) & 0x55555555u;
+#pragma unroll
+        for (int gsel = 0; gsel < 2; ++gsel) {
+            const uint32_t index = ((idx_pair >> (8 * gsel)) & 0xff) | (((qh >> (2 * gsel)) & 3) << 8);
+            const uint4 selector = codebook->entry[index];
+            const uint32_t words[4] = {selector.x, selector.y, selector.z, selector.w};
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int i = 4 * gsel + p;
+                const uint32_t picked = __builtin_amdgcn_perm(high, low_pair, words[p]);
+                pairs[i] = ((spread << (15 - 2 * i)) & 0x80008000u) | (picked & 0x7fff7fffu);
+            }
+        }
+    } else {
+        float w[16];
+        decode16_f32<TYPE>(blk, u, codebook, w);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            pairs[i] = pack_bf16x2(w[2 * i], w[2 * i + 1]);
         }
     }
 }

@@ -49,6 +49,7 @@ struct GemvArgs {
     int out_features;
     int n_groups;   // workgroups per task and projection: groups of GEMV_GN (long) weight rows
     int projections;   // 1, or 2 for a pair
+    int unit_staging;  // 2-byte aligned formats: the tensors may be read in whole aligned 16-byte units (wide_stage_ok)
 };
 
 // LDS slot of super-block `kb` of a pass for weight row `row`.  Row-major, so that the lanes of a wave, which
@@ -56,6 +57,12 @@ struct GemvArgs {
 // super-blocks outermost the stride is 16 pitches, an even number of words, and the lanes' reads of one
 // instruction pile up eight deep on a few banks.
 TGO_DEVICE int gemv_slot(int kb, int row) { return row * GEMV_CHUNK + kb; }
+// bytes per slot: the format's padded block, or the larger slot of the aligned-unit staging (gemv_stage_units)
+template <int TYPE>
+constexpr int gemv_slot_bytes() {
+    return Format<TYPE>::BLOCK_BYTES % 16 == 0 || Format<TYPE>::RAW_PITCH > WideStage<TYPE>::PITCH ? Format<TYPE>::RAW_PITCH
+                                                                                                  : WideStage<TYPE>::PITCH;
+}
 // The matrix-core variant's lanes differ in the weight row instead, and take the other order for the same reason
 // (byte offset of the slot, given its pitch).  Sixteen slots are a multiple of 16 words, and the staging writes of
 // consecutive lanes, 4 words apart within a block, would meet the same eight banks again in the next
@@ -158,6 +165,63 @@ TGO_DEVICE void gemv_stage_pieces(uint8_t * raw, const uint8_t * weights, int64_
                 }
             }
         }
+    }
+}
+
+// The same pass as aligned 16-byte units (the 2-byte aligned formats, tensors that start and end on a unit boundary:
+// wide_stage_ok): every (weight row, super-block) is covered by WideStage::UNITS aligned units, each loaded whole
+// and written to the block's slot with four 4-byte stores, shifted by the block's misalignment on the way
+// (v_alignbyte for the odd halfword, the store position for the rest), so that the block starts at
+// WideStage::FRONT of its slot.  A third of the vector instructions of dealing out 2-byte pieces.  Slots are
+// WideStage::PITCH bytes here.  `tile`: first byte of (long) weight row n0 (wave-uniform).
+template <int TYPE>
+struct GemvUnits {
+    using W = WideStage<TYPE>;
+    static constexpr int TOTAL = GEMV_GN * GEMV_CHUNK * W::UNITS;
+    static constexpr int REGS = (TOTAL + GEMV_THREADS - 1) / GEMV_THREADS;
+    static constexpr int RECIPROCAL = (65536 + W::UNITS - 1) / W::UNITS;   // id -> id / UNITS, exact below 3000
+    static_assert(TOTAL < 3000, "range of the reciprocal");
+};
+template <int TYPE>
+TGO_DEVICE void gemv_stage_units(uint8_t * raw, const uint8_t * tile, int64_t row_bytes, int rows_valid, int kb0,
+                                 int chunk_blocks, int tid) {
+    using U = GemvUnits<TYPE>;
+    using W = WideStage<TYPE>;
+    const uint32_t tile_m = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) & 15u;
+    const uint8_t * const aligned = tile - tile_m;
+    u32x4_t unit_value[U::REGS];
+    uint32_t next_value[U::REGS];
+    uint32_t place[U::REGS];   // LDS byte offset of the unit's first word | halfword shift << 16
+#pragma unroll
+    for (int i = 0; i < U::REGS; ++i) {
+        // ids past the pass repeat its last unit: no lane branches around a load
+        const int id = min(tid + GEMV_THREADS * i, U::TOTAL - 1);
+        const int slot = static_cast<int>(__umul24(id, U::RECIPROCAL) >> 16);   // gemv_slot(kb, row) = row * GEMV_CHUNK + kb
+        int unit = id - slot * W::UNITS;
+        const int row = min(slot / GEMV_CHUNK, rows_valid - 1);
+        const int kb = min(slot % GEMV_CHUNK, chunk_blocks - 1);
+        // (a pass of 16 rows spans less than 2^31 bytes: the host checks row_bytes)
+        const uint32_t first = tile_m + static_cast<uint32_t>(row) * static_cast<uint32_t>(row_bytes) +
+                               static_cast<uint32_t>(kb0 + kb) * W::BLOCK;
+        const int reach = static_cast<int>(first & 15u) + W::BLOCK;   // block end, from its first unit
+        const bool carries = 16 * (unit + 1) < reach;                 // the following unit still holds bytes of the block
+        const int source_unit = 16 * unit < reach ? unit : 0;         // (units past the block re-read its first one)
+        const uint32_t offset = (first & ~15u) + 16u * source_unit;
+        unit_value[i] = *reinterpret_cast<const u32x4_t *>(aligned + offset);
+        next_value[i] = *reinterpret_cast<const uint32_t *>(aligned + offset + (carries ? 16u : 0u));
+        const uint32_t m = first & 15u;
+        // rows and super-blocks the pass does not have are parked in their own slots (never read)
+        place[i] = static_cast<uint32_t>(slot * W::PITCH + W::FRONT + 16 * unit) - (m & 12u) + ((m & 2u) << 16);
+    }
+#pragma unroll
+    for (int i = 0; i < U::REGS; ++i) {
+        const uint32_t shift = place[i] >> 16;
+        const u32x4_t d = unit_value[i];
+        uint32_t * dst = reinterpret_cast<uint32_t *>(raw + (place[i] & 0xffffu));
+        dst[0] = __builtin_amdgcn_alignbyte(d.y, d.x, shift);
+        dst[1] = __builtin_amdgcn_alignbyte(d.z, d.y, shift);
+        dst[2] = __builtin_amdgcn_alignbyte(d.w, d.z, shift);
+        dst[3] = __builtin_amdgcn_alignbyte(next_value[i], d.w, shift);
     }
 }
 
@@ -314,7 +378,7 @@ TGO_DEVICE void gemv_unit(const uint8_t * blk, int u, const uint2 * grid, uint32
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const uint32_t nibble = (sign_pair >> (8 * gsel + 4 * h)) & 0xfu;
-                const uint32_t bits = (nibble * 0x00204081u) & 0x01010101u;   // sign bit e -> bit 0 of byte e
+                const uint32_t bits = __umul24(nibble, 0x00204081u) & 0x01010101u;   // sign bit e -> bit 0 of byte e (a 24-bit multiply: full rate)
                 const uint32_t mask = (bits << 8) - bits;                      // 0xff in the bytes to negate
                 w[2 * gsel + h] = ((h == 0 ? magnitudes.x : magnitudes.y) ^ mask) + bits;
             }
@@ -348,6 +412,10 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
     const int64_t long_row_bytes = a.row_bytes * FOLD;
     const int long_rows = a.out_features / FOLD;
     const int lane_kb = FOLD == 1 ? 0 : FOLD == 2 ? lane >> 4 : (lane >> 4) & 1;   // FOLD > 1: the lane's super-block
+    // staging by aligned units (gemv_stage_units) when the expert's tensor starts and ends on a unit boundary
+    const bool unit_staging = a.unit_staging != 0;
+    const int slot_pitch = unit_staging ? WideStage<TYPE>::PITCH : F::RAW_PITCH;
+    const int slot_front = unit_staging ? WideStage<TYPE>::FRONT : F::RAW_SHIFT;
 
     float acc[ACCS][GEMV_WAVE_ROWS][ROWS];
 #pragma unroll
@@ -390,7 +458,10 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
             load_activations(kb0, 1, early[1]);
         }
         __syncthreads();   // the previous pass is done with `raw`
-        if ((long_row_bytes & 15) == 0) {
+        if (unit_staging) {
+            gemv_stage_units<TYPE>(raw, weights + static_cast<int64_t>(n0) * long_row_bytes, long_row_bytes,
+                                   min(GEMV_GN, long_rows - n0), kb0, chunk_blocks, tid);
+        } else if ((long_row_bytes & 15) == 0) {
             gemv_stage_pieces<TYPE, 16>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
         } else if ((long_row_bytes & 3) == 0) {
             gemv_stage_pieces<TYPE, 4>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
@@ -436,7 +507,7 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
 #pragma unroll
             for (int i = 0; i < GEMV_WAVE_ROWS; ++i) {
                 const int n_local = wave * GEMV_WAVE_ROWS + i;
-                const uint8_t * blk = raw + gemv_slot(kb, n_local) * F::RAW_PITCH + F::RAW_SHIFT;
+                const uint8_t * blk = raw + gemv_slot(kb, n_local) * slot_pitch + slot_front;
                 uint32_t w[4];
                 float scale;
                 int bias;
@@ -1148,7 +1219,7 @@ template <int TYPE, int MAX_ROWS, int FOLD, bool WALK = false>
 __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a) {
     static_assert(!WALK || MAX_ROWS == GEMV_ROWS, "a walked call has full chunks");
     using F = Format<TYPE>;
-    __shared__ __attribute__((aligned(16))) uint8_t raw[GEMV_GN * GEMV_CHUNK * F::RAW_PITCH + GEMV_CHUNK * 4];
+    __shared__ __attribute__((aligned(16))) uint8_t raw[GEMV_GN * GEMV_CHUNK * gemv_slot_bytes<TYPE>() + GEMV_CHUNK * 4];
     __shared__ uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
     // float scale and min tables of the matrix-core variant: [scales, mins][wave][super-block][group of the wave's two][weight row]
     constexpr bool TABLES = (TYPE == Q4_K || TYPE == Q5_K) && MAX_ROWS > 2;
@@ -1208,7 +1279,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a
 template <int TYPE, int XROWS>
 __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_mfma_kernel(const GemvArgs a) {
     using F = Format<TYPE>;
-    __shared__ __attribute__((aligned(16))) uint8_t raw[GEMV_GN * GEMV_CHUNK * F::RAW_PITCH + GEMV_CHUNK * 4];
+    __shared__ __attribute__((aligned(16))) uint8_t raw[GEMV_GN * GEMV_CHUNK * gemv_slot_bytes<TYPE>() + GEMV_CHUNK * 4];
     __shared__ __attribute__((aligned(16))) float scale_lds[2 * (GEMV_THREADS / 64) * GEMV_CHUNK * GEMV_K45_KB_SCALES];
     __shared__ __attribute__((aligned(16))) uint8_t x_lds[XROWS * GEMV_X_PITCH + 2 * XROWS * GEMV_XD_PITCH * 4];
     const int n_group = blockIdx.x % a.n_groups;
@@ -1308,6 +1379,12 @@ hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second
     args.in_features = in_features;
     args.out_features = out_features;
     args.n_groups = (out_features + GEMV_GN - 1) / GEMV_GN;
+    // (a dense call has one "expert": the whole weight)
+    const int64_t weight_bytes = static_cast<int64_t>(out_features) * args.row_bytes;
+    args.unit_staging = block_bytes(quant_type) % 16 != 0 && wide_stage_ok(packed, weight_bytes) &&
+                                (packed_second == nullptr || wide_stage_ok(packed_second, weight_bytes)) &&
+                                args.row_bytes < (1 << 24)
+                            ? 1 : 0;
     int task_slots = 1;
     if (tasks != nullptr) {
         args.task_count = tasks->count;

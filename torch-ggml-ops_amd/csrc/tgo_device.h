@@ -829,8 +829,8 @@ TGO_DEVICE void scaled_halves(uint32_t bytes, const HalfScale & scale, uint32_t 
 
 // Values 16u .. 16u+15 of a super-block as the forward's fp16 operand: first[i] holds values 2i and 2i + 1;
 // `second` is Q6_K's low-scale operand (untouched otherwise).  Q4_K/Q5_K have their own loop in the kernel.
-template <int TYPE>
-TGO_DEVICE void decode16_half(const uint8_t * blk, int u, const uint2 * grid, uint32_t (&first)[8], uint32_t (&second)[8]) {
+template <int TYPE, typename Codebook>
+TGO_DEVICE void decode16_half(const uint8_t * blk, int u, const Codebook * grid, uint32_t (&first)[8], uint32_t (&second)[8]) {
     static_assert(TYPE == Q3_K || TYPE == Q6_K || TYPE == IQ2_S, "formats with 16-value scale groups");
     if constexpr (TYPE == Q3_K) {
         // b = low bits | high bit << 2 in 0..7, quant b - 4, operand (sc - 32) * (b - 4)
@@ -883,6 +883,29 @@ TGO_DEVICE void decode16_half(const uint8_t * blk, int u, const uint2 * grid, ui
             first[2 * t + 1] = half2_mul(q, coarse);
             second[2 * t] = half2_mul(p, fine);
             second[2 * t + 1] = half2_mul(q, fine);
+        }
+    } else if constexpr (std::is_same_v<Codebook, Iq2sSelectors>) {
+        // (the selector table of decode16_bf16: the unit's values are +-(2 s + 1) times one of three magnitudes, so
+        // three products are formed per unit and every pair of values picks its two with one byte permute)
+        const uint8_t * qs = blk + 2;
+        const uint32_t idx_pair = lds_u16(qs + 2 * u);
+        const uint32_t sign_pair = lds_u16(qs + 32 + 2 * u);
+        const uint32_t qh = blk[66 + (u >> 1)] >> (4 * (u & 1));
+        const half2_t multiplier = half2_of(2 * static_cast<int>((blk[74 + (u >> 1)] >> (4 * (u & 1))) & 0x0f) + 1);
+        const uint32_t low_pair = half2_mul(__builtin_bit_cast(uint32_t, multiplier), half2_t{static_cast<_Float16>(8.0f), static_cast<_Float16>(25.0f)});
+        const uint32_t high = half2_mul(__builtin_bit_cast(uint32_t, multiplier), half2_t{static_cast<_Float16>(43.0f), static_cast<_Float16>(0.0f)});
+        const uint32_t spread = (sign_pair & 0x5555u) | ((sign_pair & 0xaaaau) << 15);
+#pragma unroll
+        for (int gsel = 0; gsel < 2; ++gsel) {
+            const uint32_t index = ((idx_pair >> (8 * gsel)) & 0xff) | (((qh >> (2 * gsel)) & 3) << 8);
+            const uint4 selector = grid->entry[index];
+            const uint32_t words[4] = {selector.x, selector.y, selector.z, selector.w};
+#pragma unroll
+            for (int p = 0; p < 4; ++p) {
+                const int i = 4 * gsel + p;
+                const uint32_t picked = __builtin_amdgcn_perm(high, low_pair, words[p]);
+                first[i] = ((spread << (15 - 2 * i)) & 0x80008000u) | (picked & 0x7fff7fffu);
+            }
         }
     } else {
         const uint8_t * qs = blk + 2;

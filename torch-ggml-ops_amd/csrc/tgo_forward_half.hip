@@ -57,7 +57,7 @@ struct HalfLds {
     alignas(16) uint8_t wq[BUFFERS][HalfShape<TYPE>::PLANES][HalfShape<TYPE>::PLANE_BYTES];   // fp16 operand of a stage, fragment order
     alignas(16) float ws[BUFFERS][FWD_TN];                                                 // weight scale of the super-block
     alignas(16) float wm[BUFFERS][Format<TYPE>::HAS_MIN ? 8 : 1][FWD_TN];                  // block minima
-    uint2 grid[TYPE == IQ2_S ? TGO_IQ2S_GRID_ENTRIES : 1];
+    std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;   // IQ2_S: the selector table of decode16_half
 };
 
 // fp32 scale of a super-block's weight operand (decode16_half)
@@ -89,7 +89,7 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
     auto & wq = lds.wq;
     auto & ws = lds.ws;
     auto & wm = lds.wm;
-    auto & grid = lds.grid;
+    const auto * const grid = &lds.codebook;
     // (the thread id is made opaque so that a caller running two passes in a loop gets each pass compiled
     // like a lone one: nothing derived from it can be computed once and kept alive across both passes)
     int tid = threadIdx.x;
@@ -107,7 +107,7 @@ TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, in
     const int super_blocks = a.in_features / QK_K;
 
     if constexpr (TYPE == IQ2_S) {
-        expand_iq2s_grid(grid, tid, THREADS);
+        expand_iq2s_selectors(lds.codebook, tid, THREADS);
     }
 
     const int granule = NARROW ? 0 : wave;

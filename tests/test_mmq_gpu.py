@@ -69,6 +69,38 @@ def test_dequant_kernel_handles_signed_and_subnormal_scales(ops, oracle):
         np.testing.assert_array_equal(bits(out), oracle.dequant_bf16(qtype, host, k), err_msg=qname)
 
 
+@pytest.mark.parametrize("rows", (48, 300))
+@pytest.mark.parametrize("qname", tuple(QTYPES))
+def test_grad_input_decoders_handle_signed_and_subnormal_scales(ops, oracle, qname, rows):
+    """The dequantizers inside the grad-input kernels (their own code, not the dequant kernel's): random block bytes
+    with negative and subnormal fp16 super-scales, identity cotangents, so that row i of the result is weight row i
+    as the reference decoder rounds it (compared as numbers: a product's zeros lose their sign in the accumulation).
+    48 rows: the short-task kernels; 300: the others."""
+    _, native, _ = ops
+    qtype, n, k = QTYPES[qname], rows, 512
+    rng = np.random.default_rng(1234 + qtype + rows)
+    block = native.lib.tgo_block_bytes(qtype)
+    data = rng.integers(0, 256, (n * (k // 256), block), dtype=np.uint8)
+    for offset in {11: (108,), 12: (0, 2), 13: (0, 2), 14: (208,), 22: (0,)}[qtype]:
+        raw = (
+            (rng.integers(0, 2, len(data)).astype(np.uint16) << 15)
+            | (rng.integers(0, 31, len(data)).astype(np.uint16) << 10)   # exponent 0 = subnormal
+            | rng.integers(0, 1024, len(data)).astype(np.uint16)
+        )
+        data[:, offset : offset + 2] = raw.view(np.uint8).reshape(-1, 2)
+    host = data.reshape(n, -1)
+    identity = torch.eye(n, device="cuda", dtype=torch.bfloat16)
+    actual = torch.ops.torch_ggml_ops.mmq_grad_input.default(identity, torch.from_numpy(host).cuda(), qtype, k)
+    logical = oracle.bf16_to_f32(oracle.dequant_bf16(qtype, host, k))
+    np.testing.assert_array_equal(f32(actual), logical)
+    # the grouped operator takes other kernels (role-split / pipelined / short-task) than the dense one
+    experts = torch.tensor([0], device="cuda", dtype=torch.int64)
+    offsets = torch.tensor([n], device="cuda", dtype=torch.int32)
+    grouped = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default(
+        identity, torch.from_numpy(host).cuda().unsqueeze(0), experts, offsets, qtype, k)
+    np.testing.assert_array_equal(f32(grouped), logical)
+
+
 @pytest.mark.parametrize("rows,k", [(1, 256), (33, 512), (129, 2048)])
 def test_q8_1_quantizer_matches_oracle_bit_for_bit(ops, oracle, rows, k):
     _, native, _ = ops

@@ -35,7 +35,7 @@ constexpr int BWD_TK = 128;                // K columns per workgroup
 constexpr int BWD_NS = 64;                 // weight rows per reduction step
 constexpr int BWD_PITCH = BWD_NS + 8;      // bf16 per k-row of the tile: +8 keeps 16-byte reads conflict free
 constexpr int BWD_THREADS = 256;
-constexpr int BWD_XCD_RUN = 4;             // consecutive row tasks (mostly tiles of one expert) that share an XCD and its L2
+constexpr int BWD_XCD_RUN = 4;             // dense calls: consecutive row tasks that share an XCD (grouped calls: xcd_chunk)
 static_assert(BWD_TR == 64 * BWD_THREADS / 64, "64 rows per wave");
 
 // ---- cotangent packing ---------------------------------------------------------------------------------
@@ -201,11 +201,17 @@ TGO_DEVICE void decode_k45_octet(const uint8_t * raw, const float2 * scale_min, 
 }
 
 // First task and number of tasks of the list's segment that a launch runs.
-TGO_DEVICE void task_segment(const BackwardArgs & a, int & first, int & tasks) {
+// `ordinary`: how many of them come before the short ones (all of them in a segment of one kind).
+TGO_DEVICE void task_segment(const BackwardArgs & a, int & first, int & tasks, int & ordinary) {
     const int count = a.task_count[0];
-    const int early = a.task_early[0];
+    const int early = min(a.task_early[0], count);
     first = a.segment == 2 ? early : 0;
     tasks = a.segment == 2 ? count - early : a.segment == 1 ? early : count;
+    ordinary = a.segment == 0 ? early : tasks;
+}
+TGO_DEVICE void task_segment(const BackwardArgs & a, int & first, int & tasks) {
+    int ordinary;
+    task_segment(a, first, tasks, ordinary);
 }
 
 // SHORT: the variant for tasks of at most BACKWARD_SHORT_ROWS rows.  Dequantizing a step's weights costs the same
@@ -250,13 +256,17 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
     const int l32 = lane & 31;
     const int half = lane >> 5;
 
-    int k_tile, task, first_task = 0;
+    int k_tile, task, first_task = 0, ordinary = 0;
     int tasks = (a.rows + BWD_TR - 1) / BWD_TR;
     if (a.task_count != nullptr) {
-        task_segment(a, first_task, tasks);
+        task_segment(a, first_task, tasks, ordinary);
     }
-    // (short tasks are remainders of different experts: nothing to gain from runs of tasks per XCD)
-    xcd_tile<SHORT ? 1 : BWD_XCD_RUN>(blockIdx.x, a.k_tiles, tasks, k_tile, task);
+    // (short tasks are remainders of different experts: nothing to gain from keeping neighbours on one XCD)
+    if (!SHORT && a.task_count != nullptr) {
+        xcd_chunk(blockIdx.x, a.k_tiles, tasks, ordinary, k_tile, task);
+    } else {
+        xcd_tile<SHORT ? 1 : BWD_XCD_RUN>(blockIdx.x, a.k_tiles, tasks, k_tile, task);
+    }
     const int kb = k_tile >> 1;          // super-block column
     const int half_block = k_tile & 1;   // which 128 values of it
 
@@ -873,12 +883,14 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
         SplitItem item = {0, 0, 0, -1};
         const int64_t linear = blockIdx.x + static_cast<int64_t>(lane) * gridDim.x;
         if (linear < total_items) {
-            int k_tile, task, first_task = 0;
+            int k_tile, task, first_task = 0, ordinary = 0;
             int tasks = (a.rows + BWD_TR - 1) / BWD_TR;
             if (a.task_count != nullptr) {
-                task_segment(a, first_task, tasks);   // (never the short segment: first_task is 0)
+                task_segment(a, first_task, tasks, ordinary);   // (never the short segment: first_task is 0)
+                xcd_chunk(static_cast<int>(linear), a.k_tiles, tasks, ordinary, k_tile, task);
+            } else {
+                xcd_tile<BWD_XCD_RUN>(static_cast<int>(linear), a.k_tiles, tasks, k_tile, task);
             }
-            xcd_tile<BWD_XCD_RUN>(static_cast<int>(linear), a.k_tiles, tasks, k_tile, task);
             if (a.task_count != nullptr) {
                 if (task < tasks) {
                     item.expert = a.task_expert[task];
@@ -1639,7 +1651,8 @@ __global__ __launch_bounds__(256) void reduce_partials_kernel(const float * __re
 
 template <int TYPE>
 static hipError_t launch_backward_typed(const BackwardArgs & args, hipStream_t stream) {
-    const int64_t total = static_cast<int64_t>(args.k_tiles) * pad_task_slots(args.task_slots, BWD_XCD_RUN);
+    const int64_t total = static_cast<int64_t>(args.k_tiles) *
+                          (args.task_count != nullptr ? xcd_chunk_slots(args.task_slots) : pad_task_slots(args.task_slots, BWD_XCD_RUN));
     const int64_t total_short = static_cast<int64_t>(args.k_tiles) * pad_task_slots(args.short_slots);
     if (total <= 0 || total > 0x7fffffffLL || total_short > 0x7fffffffLL) {
         return hipErrorInvalidValue;

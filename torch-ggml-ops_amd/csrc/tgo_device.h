@@ -78,8 +78,8 @@ constexpr int XCDS = 8;
 
 // With fewer tasks than XCDs that grouping would leave whole XCDs idle (a dense call of up to one row tile would
 // run on an eighth of the chip), so then the tiles of a task are dealt out in plain order, i.e. across the XCDs.
-// RUN: consecutive tasks that share an XCD.  Consecutive tasks are usually row tiles of the same expert, i.e. the
-// same weights: with RUN = 1 an expert of eight or more tiles has its weights fetched into all eight L2s.
+// RUN: consecutive tasks that share an XCD.  (Dense calls and the short tasks of the grad-input; grouped launches,
+// where consecutive tasks are row tiles of the same expert, i.e. of the same weights, take xcd_chunk below.)
 template <int RUN = 1>
 TGO_DEVICE void xcd_tile(int linear, int inner, int tasks, int & inner_id, int & task) {
     if (tasks < XCDS) {
@@ -97,6 +97,35 @@ TGO_DEVICE void xcd_tile(int linear, int inner, int tasks, int & inner_id, int &
     task = (group * XCDS + (within % XCDS)) * run + run_task;
     inner_id = slot - run_task * inner;
 }
+
+// Grouped launches: consecutive tasks of the list are row tiles of the same expert, i.e. of the same weights, so
+// XCD x takes the x-th eighth of the list as one contiguous chunk and an expert's weights are fetched into one L2
+// (two where a chunk boundary cuts through it).  The chunks differ by at most one task.  A list may put cheap
+// tasks behind the others (`early` = number of ordinary ones): both parts are dealt out that way, so every XCD gets
+// its share of either kind and ends with the cheap ones.  The grid holds inner * xcd_chunk_slots(task slots)
+// workgroups; a slot past its XCD's chunks returns task = tasks.
+TGO_DEVICE void xcd_chunk(int linear, int inner, int tasks, int early, int & inner_id, int & task) {
+    if (tasks < XCDS) {
+        task = linear / inner;
+        inner_id = linear - task * inner;
+        return;
+    }
+    const int xcd = linear % XCDS;
+    const int slot = linear / XCDS;
+    int t = slot / inner;
+    inner_id = slot - t * inner;
+    const int late = tasks - early;
+    const int early_first = xcd * early / XCDS, early_end = (xcd + 1) * early / XCDS;   // (task counts stay far below 2^28)
+    const int late_first = xcd * late / XCDS, late_end = (xcd + 1) * late / XCDS;
+    if (t < early_end - early_first) {
+        task = early_first + t;
+        return;
+    }
+    t -= early_end - early_first;
+    task = t < late_end - late_first ? early + late_first + t : tasks;
+}
+
+static inline int xcd_chunk_slots(int slots) { return ((slots + XCDS - 1) / XCDS + 1) * XCDS; }
 
 static inline int pad_task_slots(int slots, int run = 1) { return (slots + XCDS * run - 1) / (XCDS * run) * (XCDS * run); }
 

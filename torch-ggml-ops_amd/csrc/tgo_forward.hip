@@ -560,7 +560,8 @@ __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_sw
 
 template <int TYPE>
 static hipError_t launch_forward_typed(const ForwardArgs & args, hipStream_t stream) {
-    const int64_t total = static_cast<int64_t>(args.n_tiles) * args.projections * pad_task_slots(args.task_slots, FWD_XCD_RUN);
+    const int64_t total = static_cast<int64_t>(args.n_tiles) * args.projections *
+                          (args.task_count != nullptr ? xcd_chunk_slots(args.task_slots) : pad_task_slots(args.task_slots, FWD_XCD_RUN));
     if (total <= 0 || total > 0x7fffffffLL) {
         return hipErrorInvalidValue;
     }
@@ -605,6 +606,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     args.n_tiles = (out_features + FWD_TN - 1) / FWD_TN;
     if (tasks != nullptr) {
         args.task_count = tasks->count;
+        args.task_early = tasks->early;
         args.task_expert = tasks->expert;
         args.task_row_start = tasks->row_start;
         args.task_row_end = tasks->row_end;
@@ -612,6 +614,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         args.dense_row_tile = forward_row_tile(quant_type, ws.half_tiles);
     } else {
         args.task_count = nullptr;
+        args.task_early = nullptr;
         args.task_expert = nullptr;
         args.task_row_start = nullptr;
         args.task_row_end = nullptr;

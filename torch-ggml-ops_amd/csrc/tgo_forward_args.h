@@ -8,7 +8,7 @@
 namespace tgo {
 
 constexpr int FWD_TN = 128;          // weight rows per workgroup
-constexpr int FWD_XCD_RUN = 4;       // consecutive row tasks (mostly tiles of one expert) that share an XCD and its L2
+constexpr int FWD_XCD_RUN = 4;       // dense calls: consecutive row tasks that share an XCD (grouped calls: xcd_chunk)
 constexpr int FWD_NT = FWD_TN / 32;  // 32-row weight tiles per workgroup
 
 struct ForwardArgs {
@@ -22,6 +22,7 @@ struct ForwardArgs {
     uint16_t * y;
     uint16_t * y_second;
     const int32_t * task_count;   // nullptr: dense
+    const int32_t * task_early;   // tasks listed before those of at most 32 rows
     const int32_t * task_expert;
     const int32_t * task_row_start;
     const int32_t * task_row_end;
@@ -42,7 +43,11 @@ TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second,
                              int & row_end) {
     int task;
     const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + a.dense_row_tile - 1) / a.dense_row_tile;
-    xcd_tile<FWD_XCD_RUN>(blockIdx.x, a.n_tiles * a.projections, tasks, n_tile, task);
+    if (a.task_count != nullptr) {
+        xcd_chunk(blockIdx.x, a.n_tiles * a.projections, tasks, min(a.task_early[0], tasks), n_tile, task);
+    } else {
+        xcd_tile<FWD_XCD_RUN>(blockIdx.x, a.n_tiles * a.projections, tasks, n_tile, task);
+    }
     second = n_tile >= a.n_tiles;
     n_tile -= second ? a.n_tiles : 0;
     expert = 0;

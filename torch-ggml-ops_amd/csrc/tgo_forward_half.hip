@@ -583,7 +583,8 @@ __global__ __launch_bounds__(HalfShape<TYPE>::THREADS, 2) void mmq_forward_half_
 
 template <int TYPE>
 static hipError_t launch_forward_half_typed(const ForwardArgs & args, hipStream_t stream) {
-    const int64_t total = static_cast<int64_t>(args.n_tiles) * args.projections * pad_task_slots(args.task_slots, FWD_XCD_RUN);
+    const int64_t total = static_cast<int64_t>(args.n_tiles) * args.projections *
+                          (args.task_count != nullptr ? xcd_chunk_slots(args.task_slots) : pad_task_slots(args.task_slots, FWD_XCD_RUN));
     if (total <= 0 || total > 0x7fffffffLL) {
         return hipErrorInvalidValue;
     }

@@ -413,9 +413,10 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
     const tgo::TaskList tasks = tgo::task_list_view(task_base, rows, num_groups, row_tile);
 
     // the quantizer writes the tile-task list on the side; the MFMA kernel runs a task of at most 32 rows in
-    // about a third of a full task's time, so those are listed last and fill the grid's tail
+    // about a third of a full task's time, so the groups of that size are listed last and fill the grid's tail
+    // (a larger group's remainder stays with the group: its weights are in that XCD's L2 already)
     const tgo::TaskBuild build = {expert_indices, expert_offsets, tasks, static_cast<int>(num_experts),
-                                  static_cast<int>(num_groups), static_cast<int>(rows), row_tile, gemv ? 0 : 32};
+                                  static_cast<int>(num_groups), static_cast<int>(rows), row_tile, gemv ? 0 : 32, 1};
     TGO_TRY(check_hip(tgo::launch_quantize_q8_1(static_cast<const uint16_t *>(input_bf16), view, rows, in_features,
                                                 hip_stream, row_index, input_rows, &build),
                       "quantize_q8_1 launch"));
@@ -529,7 +530,7 @@ static int grouped_grad_input(const void * grad_output_first, const void * grad_
     // tasks of at most BACKWARD_SHORT_ROWS rows go behind the others: a kernel variant of their own runs them
     const tgo::TaskBuild build = {expert_indices, expert_offsets, tasks, static_cast<int>(num_experts),
                                   static_cast<int>(num_groups), static_cast<int>(rows), row_tile,
-                                  tgo::BACKWARD_SHORT_ROWS};
+                                  tgo::BACKWARD_SHORT_ROWS, 0};
     TGO_TRY(check_hip(tgo::launch_pack_cotangent(static_cast<const uint16_t *>(grad_output_first),
                                                  static_cast<const uint16_t *>(grad_output_second), cotangent_first,
                                                  cotangent_second, static_cast<int>(rows),

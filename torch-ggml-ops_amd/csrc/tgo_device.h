@@ -140,6 +140,12 @@ TGO_DEVICE void build_tasks(const TaskBuild & b, int tid) {
     // Tasks of at most b.late_rows rows (a group's remainder) cost their workgroups a fraction of a full
     // task's time; they go behind all the others so that the grid's last wave of workgroups is made of the
     // short ones.  First sweep: how many tasks come before them.
+    // (late_whole_groups: only when that remainder is the whole group; the remainder of a larger group then stays
+    // behind the group's other tasks, where xcd_chunk keeps it on the XCD that already holds the expert's weights)
+    const auto listed_late = [&](int size) {
+        const int rest = size % b.row_tile;
+        return rest > 0 && rest <= b.late_rows && (b.late_whole_groups == 0 || size <= b.late_rows) ? 1 : 0;
+    };
     int early_total = 0;
     if (b.late_rows > 0) {
         int mine = 0;
@@ -149,7 +155,7 @@ TGO_DEVICE void build_tasks(const TaskBuild & b, int tid) {
             const int64_t expert64 = b.expert_indices[group];
             if (expert64 >= 0 && expert64 < b.num_experts && row_begin >= 0 && row_end > row_begin && row_end <= b.rows) {
                 const int size = row_end - row_begin;
-                mine += size / b.row_tile + (size % b.row_tile > b.late_rows ? 1 : 0);
+                mine += (size + b.row_tile - 1) / b.row_tile - listed_late(size);
             }
         }
         scan[tid] = mine;
@@ -179,8 +185,7 @@ TGO_DEVICE void build_tasks(const TaskBuild & b, int tid) {
                 expert = static_cast<int>(expert64);
                 const int size = row_end - row_begin;
                 count = (size + b.row_tile - 1) / b.row_tile;
-                const int rest = size % b.row_tile;
-                late = rest > 0 && rest <= b.late_rows ? 1 : 0;
+                late = listed_late(size);
             }
         }
         scan[tid] = count - late;

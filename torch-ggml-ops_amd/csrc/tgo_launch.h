@@ -149,6 +149,7 @@ struct TaskBuild {
     TaskList tasks;
     int num_experts, num_groups, rows, row_tile;
     int late_rows;  // tasks of at most this many rows are listed after all the others; 0: group order throughout
+    int late_whole_groups;   // 1: only groups of at most late_rows rows are listed late, not the remainders of larger ones
 };
 
 static inline TaskBuild no_task_build() {

@@ -1579,32 +1579,40 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     }
     decode(0, wb[0]);
     __syncthreads();
-#pragma unroll 1
-    for (int first = 0; first < steps; first += BSH_DEPTH) {
-#pragma unroll
-        for (int u = 0; u < BSH_DEPTH; ++u) {
-            const int step = first + u;
-            if (step < steps) {
-                const bool more = step + 1 < steps;
-                if (more) {
-                    // (this wave's decode of the current step, the last reader of its slot, is behind it in program order)
-                    park(step + 1, ring[(u + 1) % BSH_DEPTH]);
-                    request(step + 1 + BSH_DEPTH, ring[(u + 1) % BSH_DEPTH]);
-                }
-                multiply(wb[u & 1]);
-                request_cotangent(step + 1);
-                if (more) {
-                    wave_sync();
-                    if constexpr (K45) {
-                        scales(step + 1);
-                        wave_sync();
-                    }
-                    decode(step + 1, wb[(u + 1) & 1]);
-                }
-                __syncthreads();
-            }
+    // A step that has a successor: multiply its tile and prepare the next one.  The loop below holds no branch, so
+    // the compiler's wait-count bookkeeping sees every request on every path; with the last step's exceptions inside
+    // it, the paths that skip a wait made it wait for the newest requests before the matrix instructions (a whole
+    // memory round trip per step).
+    static_assert(BSH_DEPTH == 2, "tile and ring parity follow the position in the unrolled round");
+    auto advance = [&](int step, auto parity_tag) __attribute__((always_inline)) {
+        constexpr int u = decltype(parity_tag)::value;
+        // (this wave's decode of the current step, the last reader of its slot, is behind it in program order)
+        park(step + 1, ring[u ^ 1]);
+        multiply(wb[u]);
+        // both requests go out behind the matrix instructions, which wait for the previous step's cotangent only
+        request_cotangent(step + 1);
+        request(step + 1 + BSH_DEPTH, ring[u ^ 1]);
+        wave_sync();
+        if constexpr (K45) {
+            scales(step + 1);
+            wave_sync();
         }
+        decode(step + 1, wb[u ^ 1]);
+        __syncthreads();
+    };
+    int step = 0;
+#pragma unroll 1
+    for (; step + 2 <= last; step += 2) {
+        advance(step, std::integral_constant<int, 0>{});
+        advance(step + 1, std::integral_constant<int, 1>{});
     }
+    if (step < last) {   // uniform
+        advance(step, std::integral_constant<int, 0>{});
+        multiply(wb[1]);
+    } else {
+        multiply(wb[0]);
+    }
+    __syncthreads();
     // the tiles are free (every wave is past its last multiplication): the four 32-column slices of a 32-row tile
     // meet in LDS and leave as whole 256-byte rows
     constexpr int STAGE_PITCH = BWD_TK + 8;

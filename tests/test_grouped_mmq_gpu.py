@@ -265,6 +265,56 @@ def test_more_groups_than_one_listing_pass(ops, oracle, qname):
     assert_matches_f32_reference(actual, expected, accumulate_noise=2e-6)
 
 
+TASK_LAYOUTS = {
+    "seven_tasks": [33] * 7,                                   # fewer tasks than XCDs
+    "eight_tasks": [33] * 8,
+    "nine_tasks": [33] * 9,
+    "only_short": [5, 1, 32, 17, 9, 30, 2, 31, 8, 4, 3, 12, 21],       # every group is listed as a short one
+    "only_full": [128] * 19,
+    "short_behind_long": [1] * 21 + [300, 260, 140],
+    "remainders": [160, 7, 129, 33, 290, 64, 65, 1, 640, 31, 96, 257, 2, 384, 32, 97, 45],
+}
+
+
+@pytest.mark.parametrize("layout", tuple(TASK_LAYOUTS))
+@pytest.mark.parametrize("qname", ("Q5_K", "Q3_K"))
+def test_every_task_runs_once_whatever_the_list_looks_like(ops, qname, layout):
+    """Workgroups find their task through the XCD they run on: each XCD takes a contiguous share of the ordinary
+    tasks and one of the short ones.  Whatever the numbers of either kind, the joint call must give every group
+    exactly what a call with that group alone gives (same kernels, one task list of its own): a task left out
+    leaves rows unwritten, a wrong one writes other values."""
+    tgo, synth = ops
+    qtype, n, k = QTYPES[qname], 128, 512
+    sizes = TASK_LAYOUTS[layout]
+    experts = [(3 * i + 1) % len(sizes) for i in range(len(sizes))]
+    offsets = np.cumsum(sizes).tolist()
+    rows = offsets[-1]
+    _, first = _experts(synth, qtype, len(sizes), n, k, seed=410 + qtype)
+    _, second = _experts(synth, qtype, len(sizes), n, k, seed=420 + qtype)
+    x = random_bf16((rows, k), seed=99)
+    grad_first = random_bf16((rows, n), seed=98)
+    grad_second = random_bf16((rows, n), seed=97)
+    metadata = _metadata(experts, offsets)
+    out_first, out_second = tgo.grouped_mmq_pair(x, first, second, *metadata, qtype, n)
+    dx = torch.ops.torch_ggml_ops.grouped_mmq_pair_grad_input.default(grad_first, grad_second, first, second, *metadata, qtype, k)
+    dx_single = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default(grad_first, first, *metadata, qtype, k)
+    begin = 0
+    for expert, end in zip(experts, offsets):
+        # (a dense-sized call would take the decode kernels: keep the one-group calls above 4 rows per group)
+        if end - begin > 4:
+            alone = _metadata([expert], [end - begin])
+            one_first, one_second = tgo.grouped_mmq_pair(x[begin:end].clone(), first, second, *alone, qtype, n)
+            torch.testing.assert_close(out_first[begin:end], one_first, rtol=0, atol=0)
+            torch.testing.assert_close(out_second[begin:end], one_second, rtol=0, atol=0)
+            one_dx = torch.ops.torch_ggml_ops.grouped_mmq_pair_grad_input.default(
+                grad_first[begin:end].clone(), grad_second[begin:end].clone(), first, second, *alone, qtype, k)
+            assert torch.equal(dx[begin:end].view(torch.int16), one_dx.view(torch.int16))
+            one_dx = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default(grad_first[begin:end].clone(), first, *alone, qtype, k)
+            assert torch.equal(dx_single[begin:end].view(torch.int16), one_dx.view(torch.int16))
+        begin = end
+    assert torch.isfinite(out_first).all() and torch.isfinite(out_second).all() and torch.isfinite(dx).all()
+
+
 @pytest.mark.parametrize("qname", ("Q5_K",))
 def test_pair_at_benchmark_shape_per_expert(ops, oracle, qname):
     """The benchmark's per-expert shape (out_features 512, in_features 2048: eight reduction steps per source,

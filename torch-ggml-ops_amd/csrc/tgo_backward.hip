@@ -861,11 +861,15 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
     using F = Format<TYPE>;
     static_assert(TYPE == Q4_K || TYPE == Q5_K, "16-byte aligned blocks only");
     constexpr int RAW_UNITS = F::BLOCK_BYTES / 16;
+    // LDS pitch of a parked block: the block itself (a multiple of 16 bytes for these formats), so a wave's units
+    // land back to back with 16-byte writes; its readers address 16 rows at a time, which 36 or 44 words per row
+    // still spread over distinct banks
+    constexpr int BSP_RAW_PITCH = F::BLOCK_BYTES;
     constexpr int RAW_REGS = (BSP_ROWS_PER_DECODER * RAW_UNITS + 63) / 64;
     static_assert(RAW_REGS == 3, "await_loads takes three registers per step");
     constexpr int QS = TYPE == Q4_K ? 16 : 48;
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
-    __shared__ __attribute__((aligned(16))) uint8_t raw_all[4][3][BSP_ROWS_PER_DECODER * F::RAW_PITCH];
+    __shared__ __attribute__((aligned(16))) uint8_t raw_all[4][3][BSP_ROWS_PER_DECODER * BSP_RAW_PITCH];
     __shared__ float2 scale_min_all[4][2][4 * BSP_SM_PITCH];
     __shared__ __attribute__((aligned(16))) uint16_t stage_all[4][32 * (BWD_TK + 8)];
     __shared__ SplitItem items[BSP_MAX_ITEMS];
@@ -1008,8 +1012,8 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
                 const int id = min(lane + 64 * i, BSP_ROWS_PER_DECODER * RAW_UNITS - 1);
                 const int row = id / RAW_UNITS;
                 const int unit = id - row * RAW_UNITS;
-                uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
-                dst[0] = regs[i].x; dst[1] = regs[i].y; dst[2] = regs[i].z; dst[3] = regs[i].w;
+                static_assert(BSP_RAW_PITCH == RAW_UNITS * 16, "consecutive lanes write consecutive 16-byte units");
+                *reinterpret_cast<u32x4 *>(raw + row * BSP_RAW_PITCH + unit * 16) = regs[i];
             }
         };
         // Stages 2 and 3 are each split into the LDS reads and the arithmetic on what was read, so that the
@@ -1022,7 +1026,7 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
             uint32_t d_dmin, low, mid, high;   // the 16-byte block header: two halves, then 12 bytes of 6-bit fields
         };
         auto scales_fetch = [&](const uint8_t * raw) {
-            const uint8_t * blk = raw + (lane & 15) * F::RAW_PITCH;
+            const uint8_t * blk = raw + (lane & 15) * BSP_RAW_PITCH;
             ScaleInputs in;
             in.d_dmin = lds_u32(blk);
             in.low = lds_u32(blk + 4);
@@ -1066,7 +1070,7 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
                 const int n = 8 * octet + i;
-                const uint8_t * blk = raw + n * F::RAW_PITCH;
+                const uint8_t * blk = raw + n * BSP_RAW_PITCH;
                 in.qs[i] = lds_u32(blk + QS + 64 * half_block + 4 * word);
                 in.qh[i] = TYPE == Q5_K ? lds_u32(blk + 16 + position) : 0u;
                 in.sm[i] = scale_min[group_local * BSP_SM_PITCH + n];
@@ -1313,8 +1317,9 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     constexpr bool K45 = TYPE == Q4_K || TYPE == Q5_K;
     using W = WideStage<TYPE>;
     constexpr int RAW_UNITS = K45 ? F::BLOCK_BYTES / 16 : W::UNITS;
+    constexpr int BSH_RAW_PITCH = F::BLOCK_BYTES;   // Q4_K / Q5_K: as in the role-split kernel (16-byte park writes)
     constexpr int RAW_REGS = (BSH_ROWS_PER_WAVE * RAW_UNITS + 63) / 64;
-    constexpr int SLOT_PITCH = K45 ? F::RAW_PITCH : W::PITCH;
+    constexpr int SLOT_PITCH = K45 ? BSH_RAW_PITCH : W::PITCH;
     constexpr int SLOT_FRONT = K45 ? 0 : W::FRONT;
     constexpr int QS = TYPE == Q4_K ? 16 : 48;
     __shared__ __attribute__((aligned(16))) uint16_t wb[2][BWD_TK * BWD_PITCH];
@@ -1413,8 +1418,7 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
                 const int id = min(lane + 64 * i, BSH_ROWS_PER_WAVE * RAW_UNITS - 1);
                 const int row = id / RAW_UNITS;
                 const int unit = id - row * RAW_UNITS;
-                uint32_t * dst = reinterpret_cast<uint32_t *>(raw + row * F::RAW_PITCH + unit * 16);
-                dst[0] = regs.unit[i].x; dst[1] = regs.unit[i].y; dst[2] = regs.unit[i].z; dst[3] = regs.unit[i].w;
+                *reinterpret_cast<u32x4 *>(raw + row * BSH_RAW_PITCH + unit * 16) = regs.unit[i];
             }
         } else {
             const uint8_t * rows;
@@ -1432,7 +1436,7 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     auto scales = [&](int step) __attribute__((always_inline)) {
         const int n = lane & 15;
         const int group_local = lane >> 4;
-        const uint8_t * blk = raw + n * F::RAW_PITCH;
+        const uint8_t * blk = raw + n * BSH_RAW_PITCH;
         const uint32_t d_dmin = lds_u32(blk), low = lds_u32(blk + 4), mid = lds_u32(blk + 8), high = lds_u32(blk + 12);
         const int shift = 8 * group_local;
         const uint32_t b0 = (low >> shift) & 0xffu, b1 = (mid >> shift) & 0xffu, b2 = (high >> shift) & 0xffu;
@@ -1493,7 +1497,7 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
             const int n = 8 * octet + i;
-            const uint8_t * blk = raw + n * F::RAW_PITCH;
+            const uint8_t * blk = raw + n * BSH_RAW_PITCH;
             qs[i] = lds_u32(blk + QS + 64 * half_block + 4 * word);
             qh[i] = TYPE == Q5_K ? lds_u32(blk + 16 + position) : 0u;
             sm[i] = scale_min[group_local * BSH_SM_PITCH + n];

@@ -599,8 +599,12 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
 #pragma unroll
                 for (int rt = 0; rt < 2; ++rt) {
                     if (!SHORT || rt < row_tiles) {
-                        acc[rt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                            __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0);
+                        // (full-size tasks swap the operands: the lane then holds one task row and runs of four
+                        // neighbouring columns, which the epilogue stages with 8-byte LDS writes)
+                        acc[rt][kt] = SHORT ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                                  __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0)
+                                            : __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                                  bfrag, __builtin_bit_cast(v8bf, afrag[rt][s]), acc[rt][kt], 0, 0, 0);
                     }
                 }
             }
@@ -710,8 +714,10 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                             if (SHORT && rt >= row_tiles) {
                                 break;
                             }
-                            acc[rt][kt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0);
+                            acc[rt][kt] = SHORT ? __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                                      __builtin_bit_cast(v8bf, afrag[rt][s]), bfrag, acc[rt][kt], 0, 0, 0)
+                                                : __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                                                      bfrag, __builtin_bit_cast(v8bf, afrag[rt][s]), acc[rt][kt], 0, 0, 0);
                         }
                     }
                 }
@@ -759,18 +765,18 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
         return;
     }
     if (a.n_splits > 1) {
-        // fp32 partial sums straight from the accumulators: element v of a lane is row 8 (v / 4) + 4 half + v % 4,
-        // column l32 of its 32 x 32 tile, so the 32 lanes of a half-wave write 128 consecutive bytes
-        float * out = a.partial + (static_cast<int64_t>(split) * a.rows + wave_row) * a.in_features + k_tile * BWD_TK + l32;
+        // fp32 partial sums straight from the accumulators (operands swapped): a lane holds row l32 of its tile
+        // and, as elements 4 j .. 4 j + 3, the four columns from 8 j + 4 half on: 16-byte stores
+        float * out = a.partial + (static_cast<int64_t>(split) * a.rows + wave_row + l32) * a.in_features + k_tile * BWD_TK + 4 * half;
 #pragma unroll
         for (int rt = 0; rt < 2; ++rt) {
+            if (wave_row + rt * 32 + l32 < row_end) {
 #pragma unroll
-            for (int v = 0; v < 16; ++v) {
-                const int r = rt * 32 + 8 * (v >> 2) + 4 * half + (v & 3);
-                if (wave_row + r < row_end) {
+                for (int kt = 0; kt < 4; ++kt) {
 #pragma unroll
-                    for (int kt = 0; kt < 4; ++kt) {
-                        out[static_cast<int64_t>(r) * a.in_features + kt * 32] = acc[rt][kt][v];
+                    for (int j = 0; j < 4; ++j) {
+                        *reinterpret_cast<float4 *>(out + static_cast<int64_t>(rt * 32) * a.in_features + kt * 32 + 8 * j) =
+                            make_float4(acc[rt][kt][4 * j], acc[rt][kt][4 * j + 1], acc[rt][kt][4 * j + 2], acc[rt][kt][4 * j + 3]);
                     }
                 }
             }
@@ -782,8 +788,8 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
     for (int rt = 0; rt < 2; ++rt) {
         const int r0 = wave_row + rt * 32;
         if (r0 < row_end) {
-            store_rows_32x128<BWD_TK + 8, true>(stage, acc[rt], a.dx + static_cast<int64_t>(r0) * a.in_features + k_tile * BWD_TK,
-                                          a.in_features, row_end - r0, BWD_TK, lane);
+            store_rows_32x128<BWD_TK + 8, true, true>(stage, acc[rt], a.dx + static_cast<int64_t>(r0) * a.in_features + k_tile * BWD_TK,
+                                                a.in_features, row_end - r0, BWD_TK, lane);
         }
     }
     }
@@ -1251,8 +1257,10 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
                         }
 #pragma unroll
                         for (int rt = 0; rt < 2; ++rt) {
+                            // (operands swapped: the lane ends up with one task row and runs of four neighbouring
+                            // columns, which the epilogue stages with 8-byte LDS writes instead of 2-byte ones)
                             acc[rt][j & 3] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-                                __builtin_bit_cast(v8bf, cot[u][rt][j >> 2]), __builtin_bit_cast(v8bf, fragment[j]),
+                                __builtin_bit_cast(v8bf, fragment[j]), __builtin_bit_cast(v8bf, cot[u][rt][j >> 2]),
                                 acc[rt][j & 3], 0, 0, 0);
                         }
                     }
@@ -1276,7 +1284,7 @@ __global__ __launch_bounds__(BSP_THREADS, 2) void mmq_grad_input_split_kernel(co
                         for (int rt = 0; rt < 2; ++rt) {
                             const int r0 = wave_row + rt * 32;
                             if (r0 < row_end) {
-                                store_rows_32x128<BWD_TK + 8, true>(
+                                store_rows_32x128<BWD_TK + 8, true, true>(
                                     stage_all[wave], acc[rt],
                                     a.dx + static_cast<int64_t>(r0) * a.in_features + k_tile * BWD_TK, a.in_features,
                                     row_end - r0, BWD_TK, lane_here);

@@ -1599,6 +1599,8 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
     auto advance = [&](int step, auto parity_tag) __attribute__((always_inline)) {
         constexpr int u = decltype(parity_tag)::value;
         // (this wave's decode of the current step, the last reader of its slot, is behind it in program order)
+        // the chain of dependent waits goes first, the arithmetic of the decode fills in (measured: 1 %)
+        __builtin_amdgcn_s_setprio(3);
         park(step + 1, ring[u ^ 1]);
         multiply(wb[u]);
         // both requests go out behind the matrix instructions, which wait for the previous step's cotangent only
@@ -1609,6 +1611,7 @@ __global__ __launch_bounds__(BSH_THREADS, 3) void mmq_grad_input_short_kernel(co
             scales(step + 1);
             wave_sync();
         }
+        __builtin_amdgcn_s_setprio(0);
         decode(step + 1, wb[u ^ 1]);
         __syncthreads();
     };

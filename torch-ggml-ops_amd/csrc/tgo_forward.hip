@@ -239,6 +239,10 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
         *reinterpret_cast<float4 *>(&dxs[buffer][t / (S::ROWS / 4)][(t % (S::ROWS / 4)) * 4]) =
             make_float4(dx_next[0], dx_next[1], dx_next[2], dx_next[3]);
         __syncthreads();
+        // The unpack below is a chain of LDS round trips with little arithmetic; the other workgroup of the CU is
+        // usually in its scaling loop, which would fill every issue slot.  The chain's waves go first (measured:
+        // Q5_K forward 2.5 % faster, Q6_K 2.4 %, nothing for the other formats).
+        __builtin_amdgcn_s_setprio(3);
 
         // the last round re-fetches its own super-block instead of branching around the prefetch
         const int kb_next = kb + 1 < super_blocks ? kb + 1 : kb;
@@ -307,6 +311,7 @@ TGO_DEVICE void forward_task(const ForwardArgs & a, ForwardLds<TYPE> & lds, int 
                 }
             }
         }
+        __builtin_amdgcn_s_setprio(0);
         __syncthreads();
 
         if constexpr (ACTIVE) {

@@ -624,7 +624,7 @@ def main() -> None:
         help="after the timed region, run one 256 MiB device-to-device copy (a kernel of known traffic for "
         "scaling rocprofv3's FETCH_SIZE / WRITE_SIZE counters; not timed, not part of the result)",
     )
-    parser.add_argument("--operand", choices=("auto", "half", "int8"), default="auto",
+    parser.add_argument("--operand", choices=("auto", "half", "int8", "scaled"), default="auto",
                         help="matrix operands of the MFMA forward kernels: fp16 numbers holding the exact integers, int8, "
                         "or the library's default (fp16 for IQ2_S, int8 for the other formats)")
     args = parser.parse_args()
@@ -685,7 +685,7 @@ def main() -> None:
     weight_bytes = 2 * active * n * (k // 256) * _native.lib.tgo_block_bytes(w["qtype"])
 
     # the forward multiplies int8 operands, or fp16 numbers holding the same integers (the library's choice for IQ2_S)
-    half_operands = args.operand == "half" or (args.operand == "auto" and args.quant == "IQ2_S")
+    half_operands = args.operand in ("half", "scaled") or (args.operand == "auto" and args.quant == "IQ2_S")
     forward_peak = PEAK["bf16"] if half_operands else PEAK["int8"]   # fp16 and bf16 share the dense matrix peak
     # per-launch algorithmic work of each profiled kernel
     per_launch = {

@@ -252,6 +252,7 @@ int tgo_profile_read(int kernel, double * total_ms, int64_t * launches);
 #define TGO_OPERAND_INT8 0
 #define TGO_OPERAND_HALF 1
 #define TGO_OPERAND_AUTO 2
+#define TGO_OPERAND_SCALED 3
 int tgo_set_forward_operand(int operand);
 int tgo_forward_operand(void);
 

@@ -200,8 +200,10 @@ int tgo_profile_enable(int enabled) {
 }
 
 int tgo_set_forward_operand(int operand) {
-    if (operand != TGO_OPERAND_INT8 && operand != TGO_OPERAND_HALF && operand != TGO_OPERAND_AUTO) {
-        return fail(TGO_ERR_INVALID, "operand must be TGO_OPERAND_INT8, TGO_OPERAND_HALF or TGO_OPERAND_AUTO; got %d", operand);
+    if (operand != TGO_OPERAND_INT8 && operand != TGO_OPERAND_HALF && operand != TGO_OPERAND_AUTO &&
+        operand != TGO_OPERAND_SCALED) {
+        return fail(TGO_ERR_INVALID,
+                    "operand must be TGO_OPERAND_INT8, TGO_OPERAND_HALF, TGO_OPERAND_SCALED or TGO_OPERAND_AUTO; got %d", operand);
     }
     tgo::set_forward_operand_setting(operand);
     return TGO_OK;
@@ -281,7 +283,7 @@ int tgo_quantize_q8_1(const void * input_bf16, void * workspace, int64_t rows, i
     TGO_TRY(check_matmul_shape(rows, in_features, 1, TGO_TYPE_Q4_K));
     TGO_TRY(check_pointer(input_bf16, "input"));
     TGO_TRY(check_pointer(workspace, "workspace"));
-    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), 0);
+    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(0));
     return check_hip(tgo::launch_quantize_q8_1(static_cast<const uint16_t *>(input_bf16), view, rows, in_features,
                                                static_cast<hipStream_t>(stream)),
                      "quantize_q8_1 launch");
@@ -295,7 +297,7 @@ int tgo_q8_workspace_unpack(const void * workspace, void * q_int8, void * d_f32,
         return fail(TGO_ERR_INVALID, "output pointers must not be null");
     }
     const tgo::Q8Workspace view =
-        tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), 0);
+        tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(0));
     return check_hip(tgo::launch_q8_unpack(view, static_cast<int8_t *>(q_int8), static_cast<float *>(d_f32),
                                            static_cast<float *>(sum_f32), rows, in_features,
                                            static_cast<hipStream_t>(stream)),
@@ -310,7 +312,7 @@ int tgo_mmq_forward(const void * input_bf16, const void * packed, void * output_
     TGO_TRY(check_pointer(output_bf16, "output"));
     TGO_TRY(check_pointer(workspace, "workspace"));
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
-    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), quant_type);
+    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(quant_type));
     TGO_TRY(check_hip(tgo::launch_quantize_q8_1(static_cast<const uint16_t *>(input_bf16), view, rows, in_features,
                                                 hip_stream),
                       "quantize_q8_1 launch"));
@@ -348,7 +350,7 @@ int tgo_mmq_forward_prepared(const void * workspace, const void * packed, void *
     TGO_TRY(check_pointer(packed, "packed_weight"));
     TGO_TRY(check_pointer(output_bf16, "output"));
     const tgo::Q8Workspace view =
-        tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), 0);
+        tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(0));
     const auto launch = tgo::use_gemv(rows, 0) ? tgo::launch_mmq_gemv : tgo::launch_mmq_forward;
     return check_hip(launch(static_cast<const uint8_t *>(packed), nullptr, 0, view,
                             static_cast<uint16_t *>(output_bf16), nullptr, nullptr, static_cast<int>(rows),
@@ -406,9 +408,14 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
     const int64_t bytes_per_expert = out_features * (in_features / tgo::QK_K) * tgo::block_bytes(quant_type);
     // (the fused SwiGLU epilogue exists in the MFMA kernel only)
     const bool gemv = !swiglu && tgo::use_gemv(rows, num_groups);
-    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, gemv, quant_type);
+    // (the scaled-operand kernel has no fused SwiGLU epilogue)
+    int operand_kind = tgo::forward_operand_kind(quant_type);
+    if (swiglu && operand_kind == tgo::OPERAND_SCALED) {
+        operand_kind = quant_type == TGO_TYPE_IQ2_S ? tgo::OPERAND_HALF : tgo::OPERAND_INT8;
+    }
+    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, gemv, operand_kind);
     void * task_base = static_cast<char *>(workspace) + (tgo::q8_workspace_bytes(rows, in_features) + 15) / 16 * 16;
-    const int row_tile = gemv ? tgo::GEMV_ROW_TILE : tgo::forward_row_tile(quant_type, view.half_tiles);
+    const int row_tile = gemv ? tgo::GEMV_ROW_TILE : tgo::forward_row_tile(quant_type, view.operand_kind());
     const auto launch = swiglu ? tgo::launch_mmq_forward_swiglu : gemv ? tgo::launch_mmq_gemv : tgo::launch_mmq_forward;
     const tgo::TaskList tasks = tgo::task_list_view(task_base, rows, num_groups, row_tile);
 

@@ -89,8 +89,9 @@ TGO_DEVICE int round_magnitude(float v) {
 typedef short short2_t __attribute__((ext_vector_type(2)));
 // `halves`: the same quants as fp16 numbers, two per register (1024 + magnitude is the magnitude placed under the
 // bits of 1024.0; the sign bit is the one of the bf16 value, which sits at the same place of its half-word).
+// `magnitude`: |q| of the eight values (for the scaled layout, which stores d * q instead of q).
 TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (&packed)[2], float & d, float & total,
-                               uint32_t (&halves)[4]) {
+                               uint32_t (&halves)[4], int (&magnitude)[8]) {
     float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fabsf(x[2]));
     amax = fmaxf(fmaxf(amax, fabsf(x[3])), fabsf(x[4]));
     amax = fmaxf(fmaxf(amax, fabsf(x[5])), fabsf(x[6]));
@@ -112,8 +113,9 @@ TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (
     uint32_t signed_pairs[4];
 #pragma unroll
     for (int pair = 0; pair < 4; ++pair) {
-        const short2_t magnitudes = __builtin_amdgcn_cvt_pk_i16(round_magnitude(x[2 * pair] * d_inv),
-                                                                round_magnitude(x[2 * pair + 1] * d_inv));
+        magnitude[2 * pair] = round_magnitude(x[2 * pair] * d_inv);
+        magnitude[2 * pair + 1] = round_magnitude(x[2 * pair + 1] * d_inv);
+        const short2_t magnitudes = __builtin_amdgcn_cvt_pk_i16(magnitude[2 * pair], magnitude[2 * pair + 1]);
         const short2_t sign = __builtin_bit_cast(short2_t, words[pair]) >> 15;
         signed_pairs[pair] = __builtin_bit_cast(uint32_t, static_cast<short2_t>((magnitudes ^ sign) - sign));
         halves[pair] = half2_add(__builtin_bit_cast(uint32_t, magnitudes) | 0x64006400u, half2_of(-1024)) |
@@ -137,9 +139,13 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
                                                                 float * __restrict__ d_out,
                                                                 float * __restrict__ sum_out, int in_features,
                                                                 const int64_t * __restrict__ gather,
-                                                                int64_t input_rows, const TaskBuild build) {
+                                                                int64_t input_rows, uint32_t * __restrict__ tag,
+                                                                const TaskBuild build) {
     if (build.tasks.count != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
         build_tasks(build, threadIdx.x);
+    }
+    if (blockIdx.x == 0 && blockIdx.y == 0 && threadIdx.x == 0) {
+        *tag = WORKSPACE_TAG_MAGIC | LAYOUT_ROWS;
     }
     const int row = blockIdx.x;
     const int k = (blockIdx.y * 256 + threadIdx.x) * 8;
@@ -159,8 +165,9 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
     float x[8];
     unpack_bf16x8(bits, x);
     uint32_t packed[2], halves[4];
+    int magnitude[8];
     float d, total;
-    quantize_eight(bits, x, packed, d, total, halves);
+    quantize_eight(bits, x, packed, d, total, halves, magnitude);
     *reinterpret_cast<uint2 *>(q_out + static_cast<int64_t>(row) * in_features + k) = make_uint2(packed[0], packed[1]);
     if ((threadIdx.x & 3) == 0) {
         const int64_t block = static_cast<int64_t>(row) * (in_features / 32) + k / 32;
@@ -169,25 +176,32 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
     }
 }
 
-// HALF: the quants leave as fp16 numbers for the fp16-operand forward kernels, 16 KiB per workgroup: per 32-value
-// block two 1 KiB slabs (k-halves of 16 values), each 64 pieces of eight values = (eighth of the k-half, row).
-template <bool HALF>
+// LAYOUT_HALF_TILES: the quants leave as fp16 numbers for the fp16-operand forward kernels, 16 KiB per workgroup:
+// per 32-value block two 1 KiB slabs (k-halves of 16 values), each 64 pieces of eight values = (eighth of the
+// k-half, row).
+template <int LAYOUT>
 __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __restrict__ input,
                                                            int8_t * __restrict__ q_out,
                                                            float * __restrict__ d_out,
-                                                           float * __restrict__ sum_out, int rows,
+                                                           float * __restrict__ sum_out,
+                                                           uint32_t * __restrict__ tag, int rows,
                                                            int in_features,
                                                            const int64_t * __restrict__ gather,
                                                            int64_t input_rows, const TaskBuild build) {
+    constexpr bool WIDE_VALUES = LAYOUT != LAYOUT_INT8_TILES;   // two bytes per value
+    static_assert(LAYOUT == LAYOUT_INT8_TILES || LAYOUT == LAYOUT_HALF_TILES, "the scaled layout has a kernel of its own");
     if (build.tasks.count != nullptr && blockIdx.x == 0 && blockIdx.y == 0) {
         build_tasks(build, threadIdx.x);
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        *tag = WORKSPACE_TAG_MAGIC | LAYOUT;
     }
     // Workgroups that are launched together take neighbouring column chunks of the same 32 rows, so that what the
     // chip reads and writes at any time are whole rows and 8 KiB fragment runs next to each other (with the row
     // tiles of one chunk launched together instead, the same kernel ran at 4.8 instead of 5.9 TB/s).
     const int chunks = in_features / 256;
     const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
-    __shared__ __attribute__((aligned(16))) uint8_t tile[(HALF ? 16 : 8) * 1024];
+    __shared__ __attribute__((aligned(16))) uint8_t tile[(WIDE_VALUES ? 16 : 8) * 1024];
     __shared__ __attribute__((aligned(16))) float scales[2][8][32];   // d and sum of the tile: [which][block][row]
     const int tid = threadIdx.x;
     const int row_tile = blockIdx.x / chunks;                 // 32-row tile
@@ -228,10 +242,11 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
         const uint4 row_bits = present[pass] ? bits[pass] : uint4{0, 0, 0, 0};
         unpack_bf16x8(row_bits, x);
         uint32_t packed[2], halves[4];
+        int magnitude[8];
         float d, total;
-        quantize_eight(row_bits, x, packed, d, total, halves);
+        quantize_eight(row_bits, x, packed, d, total, halves, magnitude);
         const int half = quarter >> 1;
-        if constexpr (HALF) {
+        if constexpr (WIDE_VALUES) {
             // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
             *reinterpret_cast<uint4 *>(tile + block * 2048 + half * 1024 + (rr + 32 * (quarter & 1)) * 16) =
                 make_uint4(halves[0], halves[1], halves[2], halves[3]);
@@ -252,7 +267,7 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
         *reinterpret_cast<float4 *>(plane + static_cast<int64_t>(chunk * 8 + b) * rows_padded + row_tile * 32 + piece * 4) =
             *reinterpret_cast<const float4 *>(&scales[which][b][piece * 4]);
     }
-    constexpr int BLOCK_BYTES = HALF ? 2048 : 1024;
+    constexpr int BLOCK_BYTES = WIDE_VALUES ? 2048 : 1024;
     uint4 * dst = reinterpret_cast<uint4 *>(
         q_out + (static_cast<int64_t>(row_tile) * blocks_per_row + chunk * 8) * BLOCK_BYTES);
     const uint4 * src = reinterpret_cast<const uint4 *>(tile);
@@ -262,15 +277,196 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
     }
 }
 
+// LAYOUT_SCALED_TILES: the fp16 slabs of the half layout hold the dequantized values d * q instead of q, normalised
+// per row by the power of two 2^E that brings the row's largest magnitude into [2^8, 2^9), and rounded once to
+// fp16 (relative 2^-12); 2^E goes to the `power` plane, one number per row, and the block sums, scaled alike, to
+// `block_sums` as fp16, eight per row and super-block: the operand that meets the block minima of Q4_K/Q5_K.  The
+// scale and sum planes are written as in every layout.  The exponent needs the whole row, so a workgroup takes 32
+// rows x all of K: a first pass finds the rows' maxima, a second one quantizes chunk by chunk.  RESIDENT (K up to
+// 2048): the rows stay in registers between the passes; otherwise the second pass reads them again.
+template <bool RESIDENT>
+__global__ __launch_bounds__(256) void quantize_q8_1_scaled_kernel(const uint16_t * __restrict__ input,
+                                                                  int8_t * __restrict__ q_out,
+                                                                  float * __restrict__ d_out,
+                                                                  float * __restrict__ sum_out,
+                                                                  float * __restrict__ power_out,
+                                                                  uint16_t * __restrict__ block_sums_out,
+                                                                  uint32_t * __restrict__ tag, int rows,
+                                                                  int in_features,
+                                                                  const int64_t * __restrict__ gather,
+                                                                  int64_t input_rows, const TaskBuild build) {
+    if (build.tasks.count != nullptr && blockIdx.x == 0) {
+        build_tasks(build, threadIdx.x);
+    }
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        *tag = WORKSPACE_TAG_MAGIC | LAYOUT_SCALED_TILES;
+    }
+    constexpr int GROUP = 8;   // chunks of 256 values whose loads are in flight together
+    const int chunks = in_features / 256;
+    const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
+    __shared__ __attribute__((aligned(16))) uint8_t tile[16 * 1024];
+    __shared__ __attribute__((aligned(16))) float scales[2][8][32];   // d and sum of the chunk: [which][block][row]
+    __shared__ __attribute__((aligned(16))) uint16_t sums_half[32][8];
+    __shared__ __attribute__((aligned(16))) float powers[32];
+    const int tid = threadIdx.x;
+    const int row_tile = blockIdx.x;
+    const int blocks_per_row = in_features / 32;
+    const int lane_k = tid & 31;       // 8 values each
+    const int block = lane_k >> 2;     // 32-value block inside the chunk
+    const int quarter = lane_k & 3;
+
+    int64_t source[4];
+    bool present[4];
+    const int last_row = rows - 1;
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        const int row = row_tile * 32 + (tid >> 5) + 8 * pass;
+        present[pass] = row < rows;
+        source[pass] = min(row, last_row);
+        if (gather != nullptr) {   // uniform
+            source[pass] = gather[source[pass]];
+            present[pass] = present[pass] && source[pass] >= 0 && source[pass] < input_rows;
+            source[pass] = present[pass] ? source[pass] : 0;
+        }
+    }
+    auto load_chunk = [&](int chunk, uint4 (&bits)[4]) {
+        const int clamped = min(chunk, chunks - 1);
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            bits[pass] = *reinterpret_cast<const uint4 *>(input + source[pass] * in_features + clamped * 256 + lane_k * 8);
+            if (!present[pass] || chunk >= chunks) {
+                bits[pass] = uint4{0, 0, 0, 0};
+            }
+        }
+    };
+    // ---- first pass: the largest magnitude of each of the thread's four rows
+    uint4 resident[RESIDENT ? GROUP : 1][4];
+    float largest[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    for (int first = 0; first < chunks; first += GROUP) {
+        uint4 group[GROUP][4];
+#pragma unroll
+        for (int c = 0; c < GROUP; ++c) {
+            load_chunk(first + c, group[c]);
+        }
+#pragma unroll
+        for (int c = 0; c < GROUP; ++c) {
+#pragma unroll
+            for (int pass = 0; pass < 4; ++pass) {
+                float x[8];
+                unpack_bf16x8(group[c][pass], x);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    largest[pass] = fmaxf(largest[pass], fabsf(x[i]));
+                }
+                if constexpr (RESIDENT) {
+                    resident[c][pass] = group[c][pass];
+                }
+            }
+        }
+    }
+    float inverse[4];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        float amax = largest[pass];
+#pragma unroll
+        for (int offset = 1; offset < 32; offset <<= 1) {
+            amax = fmaxf(amax, __shfl_xor(amax, offset));
+        }
+        int exponent = static_cast<int>(__float_as_uint(amax) >> 23);   // biased
+        exponent = min(max(exponent, 9), 254);
+        inverse[pass] = __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-E
+        if (lane_k == 0) {
+            powers[(tid >> 5) + 8 * pass] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^E
+        }
+    }
+    __syncthreads();
+    if (tid < 8) {
+        *reinterpret_cast<float4 *>(power_out + row_tile * 32 + tid * 4) = *reinterpret_cast<const float4 *>(&powers[tid * 4]);
+    }
+    // ---- second pass: quantize, chunk by chunk
+    auto quantize_chunk = [&](int chunk, const uint4 (&bits)[4]) {
+#pragma unroll
+        for (int pass = 0; pass < 4; ++pass) {
+            const int rr = (tid >> 5) + 8 * pass;
+            float x[8];
+            unpack_bf16x8(bits[pass], x);
+            uint32_t packed[2], halves[4];
+            int magnitude[8];
+            float d, total;
+            quantize_eight(bits[pass], x, packed, d, total, halves, magnitude);
+            const float lane_scale = d * inverse[pass];
+            const uint32_t words[4] = {bits[pass].x, bits[pass].y, bits[pass].z, bits[pass].w};
+#pragma unroll
+            for (int pair = 0; pair < 4; ++pair) {
+                const half2_t values = {static_cast<_Float16>(static_cast<float>(magnitude[2 * pair]) * lane_scale),
+                                        static_cast<_Float16>(static_cast<float>(magnitude[2 * pair + 1]) * lane_scale)};
+                halves[pair] = __builtin_bit_cast(uint32_t, values) | (words[pair] & 0x80008000u);
+            }
+            // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
+            *reinterpret_cast<uint4 *>(tile + block * 2048 + (quarter >> 1) * 1024 + (rr + 32 * (quarter & 1)) * 16) =
+                make_uint4(halves[0], halves[1], halves[2], halves[3]);
+            if (quarter == 0) {
+                scales[0][block][rr] = d;
+                scales[1][block][rr] = total;
+                sums_half[rr][block] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(total * inverse[pass]));
+            }
+        }
+        __syncthreads();
+        if (tid < 128) {
+            const int which = tid >> 6, b = (tid >> 3) & 7, piece = tid & 7;
+            float * plane = which == 0 ? d_out : sum_out;
+            *reinterpret_cast<float4 *>(plane + static_cast<int64_t>(chunk * 8 + b) * rows_padded + row_tile * 32 + piece * 4) =
+                *reinterpret_cast<const float4 *>(&scales[which][b][piece * 4]);
+        } else if (tid >= 192 && tid < 224) {
+            const int row = tid - 192;
+            *reinterpret_cast<uint4 *>(block_sums_out + ((static_cast<int64_t>(row_tile) * chunks + chunk) * 32 + row) * 8) =
+                *reinterpret_cast<const uint4 *>(&sums_half[row][0]);
+        }
+        uint4 * dst = reinterpret_cast<uint4 *>(q_out + (static_cast<int64_t>(row_tile) * blocks_per_row + chunk * 8) * 2048);
+        const uint4 * src = reinterpret_cast<const uint4 *>(tile);
+#pragma unroll
+        for (int piece = 0; piece < 4; ++piece) {
+            dst[tid + 256 * piece] = src[tid + 256 * piece];
+        }
+        __syncthreads();
+    };
+    if constexpr (RESIDENT) {
+#pragma unroll
+        for (int c = 0; c < GROUP; ++c) {
+            if (c < chunks) {   // uniform
+                quantize_chunk(c, resident[c]);
+            }
+        }
+    } else {
+        for (int c = 0; c < chunks; ++c) {
+            uint4 bits[4];
+            load_chunk(c, bits);
+            quantize_chunk(c, bits);
+        }
+    }
+}
+
 hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, int64_t rows,
                                 int64_t in_features, hipStream_t stream, const int64_t * gather,
                                 int64_t input_rows, const TaskBuild * build) {
     const ProfileScope scope(0, stream);
     const TaskBuild on_the_side = build != nullptr ? *build : no_task_build();
-    if (ws.by_rows) {
+    if (ws.by_rows()) {
         const dim3 grid(static_cast<unsigned>(rows), static_cast<unsigned>((in_features + 2047) / 2048));
         quantize_q8_1_rows_kernel<<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(in_features),
-                                                            gather, input_rows, on_the_side);
+                                                            gather, input_rows, ws.tag, on_the_side);
+        return hipGetLastError();
+    }
+    const int r = static_cast<int>(rows), k = static_cast<int>(in_features);
+    if (ws.scaled_tiles()) {
+        const dim3 grid(static_cast<unsigned>(ws.rows_padded / 32));
+        if (in_features <= 2048) {
+            quantize_q8_1_scaled_kernel<true><<<grid, 256, 0, stream>>>(
+                input, ws.q, ws.d, ws.sum, ws.power, ws.block_sums, ws.tag, r, k, gather, input_rows, on_the_side);
+        } else {
+            quantize_q8_1_scaled_kernel<false><<<grid, 256, 0, stream>>>(
+                input, ws.q, ws.d, ws.sum, ws.power, ws.block_sums, ws.tag, r, k, gather, input_rows, on_the_side);
+        }
         return hipGetLastError();
     }
     const int64_t workgroups = ws.rows_padded / 32 * (in_features / 256);
@@ -278,52 +474,74 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
         return hipErrorInvalidValue;
     }
     const dim3 grid(static_cast<unsigned>(workgroups));
-    if (ws.half_tiles) {
-        quantize_q8_1_kernel<true><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(rows),
-                                                             static_cast<int>(in_features), gather, input_rows, on_the_side);
+    if (ws.half_tiles()) {
+        quantize_q8_1_kernel<LAYOUT_HALF_TILES><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, ws.tag, r, k, gather,
+                                                                           input_rows, on_the_side);
     } else {
-        quantize_q8_1_kernel<false><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, static_cast<int>(rows),
-                                                              static_cast<int>(in_features), gather, input_rows, on_the_side);
+        quantize_q8_1_kernel<LAYOUT_INT8_TILES><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, ws.tag, r, k, gather,
+                                                                           input_rows, on_the_side);
     }
     return hipGetLastError();
 }
 
+// Workspace inspection for tests: the quants, scales and sums as plain rows, whichever layout the quantizer wrote
+// (read from the workspace's tag; a workspace without a valid tag yields zeros).  The scaled layout stores d * q:
+// its quants are recovered as round(value * 2^E / d), exact because the fp16 rounding moves a value by less than
+// 127 * 2^-12 of a quant step (values that the normalisation pushed below the fp16 range come back as zero).
 __global__ __launch_bounds__(256) void q8_unpack_kernel(const int8_t * __restrict__ q_frag,
                                                        const float * __restrict__ d_in,
                                                        const float * __restrict__ sum_in,
+                                                       const float * __restrict__ power_in,
+                                                       const uint32_t * __restrict__ tag,
                                                        int8_t * __restrict__ q, float * __restrict__ d,
                                                        float * __restrict__ sum, int rows,
-                                                       int in_features, bool by_rows, bool half_tiles) {
+                                                       int in_features) {
     const int64_t index = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     const int64_t total = static_cast<int64_t>(rows) * in_features;
     if (index >= total) {
         return;
     }
+    const uint32_t word = *tag;
+    const int layout = (word & 0xffff0000u) == WORKSPACE_TAG_MAGIC ? static_cast<int>(word & 0xffffu) : -1;
     const int row = static_cast<int>(index / in_features);
     const int k = static_cast<int>(index % in_features);
     const int blocks_per_row = in_features / 32;
     const int block = k >> 5, half = (k >> 4) & 1, byte = k & 15;
-    if (by_rows) {
-        q[index] = q_frag[index];
+    const int64_t block_index = static_cast<int64_t>(row) * blocks_per_row + block;
+    if (layout < 0 || layout > LAYOUT_SCALED_TILES) {
+        q[index] = 0;
         if ((k & 31) == 0) {
-            d[static_cast<int64_t>(row) * blocks_per_row + block] = d_in[static_cast<int64_t>(row) * blocks_per_row + block];
-            sum[static_cast<int64_t>(row) * blocks_per_row + block] = sum_in[static_cast<int64_t>(row) * blocks_per_row + block];
+            d[block_index] = 0.0f;
+            sum[block_index] = 0.0f;
         }
         return;
     }
-    if (half_tiles) {
-        const _Float16 * values = reinterpret_cast<const _Float16 *>(q_frag);
-        q[index] = static_cast<int8_t>(static_cast<float>(
-            values[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 + half * 512 +
-                   ((row & 31) + 32 * (byte >> 3)) * 8 + (byte & 7)]));
-    } else {
+    if (layout == LAYOUT_ROWS) {
+        q[index] = q_frag[index];
+        if ((k & 31) == 0) {
+            d[block_index] = d_in[block_index];
+            sum[block_index] = sum_in[block_index];
+        }
+        return;
+    }
+    const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
+    const float scale = d_in[block * rows_padded + row];
+    if (layout == LAYOUT_INT8_TILES) {
         q[index] = q_frag[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 +
                           ((row & 31) + 32 * half) * 16 + byte];
+    } else {
+        const _Float16 * values = reinterpret_cast<const _Float16 *>(q_frag);
+        float value = static_cast<float>(
+            values[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 + half * 512 +
+                   ((row & 31) + 32 * (byte >> 3)) * 8 + (byte & 7)]);
+        if (layout == LAYOUT_SCALED_TILES) {
+            value = scale == 0.0f ? 0.0f : rintf(value * power_in[row] / scale);
+        }
+        q[index] = static_cast<int8_t>(value);
     }
     if ((k & 31) == 0) {
-        const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
-        d[static_cast<int64_t>(row) * blocks_per_row + block] = d_in[block * rows_padded + row];
-        sum[static_cast<int64_t>(row) * blocks_per_row + block] = sum_in[block * rows_padded + row];
+        d[block_index] = scale;
+        sum[block_index] = sum_in[block * rows_padded + row];
     }
 }
 
@@ -331,7 +549,7 @@ hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float
                             int64_t in_features, hipStream_t stream) {
     const int64_t total = rows * in_features;
     q8_unpack_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(
-        ws.q, ws.d, ws.sum, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features), ws.by_rows, ws.half_tiles);
+        ws.q, ws.d, ws.sum, ws.power, ws.tag, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features));
     return hipGetLastError();
 }
 

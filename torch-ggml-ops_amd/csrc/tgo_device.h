@@ -966,6 +966,20 @@ TGO_DEVICE void decode16_half(const uint8_t * blk, int u, const Codebook * grid,
     }
 }
 
+// fp32 scale of a super-block's weight operand (decode16_half)
+template <int TYPE>
+TGO_DEVICE float half_weight_scale(const uint8_t * blk) {
+    if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
+        return half_bits_to_float(lds_u16(blk));
+    } else if constexpr (TYPE == Q3_K) {
+        return half_bits_to_float(lds_u16(blk + 108));
+    } else if constexpr (TYPE == Q6_K) {
+        return half_bits_to_float(lds_u16(blk + 208));
+    } else {
+        return half_bits_to_float(lds_u16(blk)) * 0.125f;
+    }
+}
+
 // fp32 scale (and min) of 32-value block b (0..7) of a super-block for the forward algebra.
 template <int TYPE>
 TGO_DEVICE void forward_block_scale(const uint8_t * blk, int b, float & scale, float & minimum) {

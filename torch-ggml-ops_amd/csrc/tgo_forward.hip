@@ -529,7 +529,7 @@ __global__ __launch_bounds__(ForwardShape<TYPE>::THREADS, 2) void mmq_forward_ke
     using F = Format<TYPE>;
     using S = ForwardShape<TYPE>;
     constexpr int PLANES = F::PLANES;
-    static_assert(S::ROWS == forward_row_tile(TYPE, false), "task rows match the workgroup");
+    static_assert(S::ROWS == forward_row_tile(TYPE, OPERAND_INT8), "task rows match the workgroup");
     __shared__ ForwardLds<TYPE> lds;
 
     int n_tile, expert, row_start, row_end;
@@ -583,7 +583,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
                                  const Q8Workspace & ws, uint16_t * output, uint16_t * output_second,
                                  const TaskList * tasks, int rows, int in_features, int out_features,
                                  int quant_type, hipStream_t stream, bool swiglu) {
-    if (ws.by_rows) {
+    if (ws.by_rows()) {
         return hipErrorInvalidValue;   // this kernel reads the tile-ordered activation layout
     }
     if (ws.rows_padded >= (1 << 24) || in_features >= (1 << 24)) {
@@ -603,6 +603,8 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     args.qx = ws.q;
     args.dx = ws.d;
     args.sx = ws.sum;
+    args.power = ws.power;
+    args.block_sums = ws.block_sums;
     args.y = output;
     args.rows = rows;
     args.rows_padded = static_cast<int>(ws.rows_padded);
@@ -616,7 +618,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         args.task_row_start = tasks->row_start;
         args.task_row_end = tasks->row_end;
         args.task_slots = tasks->max_tasks;
-        args.dense_row_tile = forward_row_tile(quant_type, ws.half_tiles);
+        args.dense_row_tile = forward_row_tile(quant_type, ws.operand_kind());
     } else {
         args.task_count = nullptr;
         args.task_early = nullptr;
@@ -629,7 +631,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         // but their eight waves own 32 rows each: with tiles of 128, 64 or 32 rows only 4, 2 or 1 of them multiply
         // (the others still help to unpack), the vector work of a tile no longer queues two waves deep on every
         // SIMD, and there are 2, 4 or 8 times the workgroups; the largest tile that yields 128 workgroups is taken.
-        int row_tile = forward_row_tile(quant_type, ws.half_tiles);
+        int row_tile = forward_row_tile(quant_type, ws.operand_kind());
         const auto tiles = [&](int tile) { return static_cast<int64_t>(args.n_tiles) * ((rows + tile - 1) / tile); };
         if (row_tile == 128) {
             if (tiles(128) <= 128) {
@@ -643,7 +645,10 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
         args.dense_row_tile = row_tile;
         args.task_slots = (rows + row_tile - 1) / row_tile;
     }
-    if (ws.half_tiles) {
+    if (ws.scaled_tiles()) {
+        return launch_forward_scaled(args, quant_type, stream);
+    }
+    if (ws.half_tiles()) {
         return launch_forward_half(args, quant_type, stream);
     }
     switch (quant_type) {

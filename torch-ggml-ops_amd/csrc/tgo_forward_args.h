@@ -1,4 +1,4 @@
-// What the two forward kernel families (int8 and fp16 matrix operands) share: the launch arguments and the
+// What the forward kernel families (int8, exact fp16 and scaled fp16 matrix operands) share: the launch arguments and the
 // mapping from a workgroup to its (column tile, projection, row task).
 #pragma once
 
@@ -16,9 +16,11 @@ struct ForwardArgs {
     const uint8_t * packed_second;   // second projection of a pair, or nullptr
     int64_t bytes_per_expert;
     int64_t row_bytes;
-    const int8_t * qx;               // int8 tiles, or fp16 tiles (Q8Workspace::half_tiles)
+    const int8_t * qx;               // int8 tiles, or fp16 tiles (Q8Workspace::layout)
     const float * dx;
     const float * sx;
+    const float * power;             // scaled tiles only: 2^e per row and super-block
+    const uint16_t * block_sums;     // scaled tiles only: fp16 block sums, eight per row and super-block
     uint16_t * y;
     uint16_t * y_second;
     const int32_t * task_count;   // nullptr: dense
@@ -70,5 +72,6 @@ TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second,
 
 // Launch of the fp16-operand kernels for arguments prepared by the common launcher (tgo_forward.hip).
 hipError_t launch_forward_half(const ForwardArgs & args, int quant_type, hipStream_t stream);
+hipError_t launch_forward_scaled(const ForwardArgs & args, int quant_type, hipStream_t stream);
 
 }  // namespace tgo

@@ -60,20 +60,6 @@ struct HalfLds {
     std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;   // IQ2_S: the selector table of decode16_half
 };
 
-// fp32 scale of a super-block's weight operand (decode16_half)
-template <int TYPE>
-TGO_DEVICE float half_weight_scale(const uint8_t * blk) {
-    if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
-        return half_bits_to_float(lds_u16(blk));
-    } else if constexpr (TYPE == Q3_K) {
-        return half_bits_to_float(lds_u16(blk + 108));
-    } else if constexpr (TYPE == Q6_K) {
-        return half_bits_to_float(lds_u16(blk + 208));
-    } else {
-        return half_bits_to_float(lds_u16(blk)) * 0.125f;
-    }
-}
-
 // NARROW: a task of at most 32 rows; every wave takes the same 32 activation rows and weight tile number `wave`.
 template <int TYPE, bool NARROW, bool WIDE>
 TGO_DEVICE void forward_half_task(const ForwardArgs & a, HalfLds<TYPE> & lds, int n_tile, bool second, int expert,

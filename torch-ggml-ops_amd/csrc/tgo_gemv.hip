@@ -1360,7 +1360,7 @@ hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second
                            const Q8Workspace & ws, uint16_t * output, uint16_t * output_second,
                            const TaskList * tasks, int rows, int in_features, int out_features,
                            int quant_type, hipStream_t stream) {
-    if (!ws.by_rows) {
+    if (!ws.by_rows()) {
         return hipErrorInvalidValue;   // these kernels read the row-major activation layout
     }
     GemvArgs args;

@@ -6,29 +6,47 @@
 
 namespace tgo {
 
-// Row tile of one forward / grad-input task; the task list is built for these.
-// Forward with int8 operands: 256 rows for the formats whose weights unpack into two int8 planes (Q6_K = 14,
-// IQ2_S = 22), 128 rows for the single-plane ones; with fp16 operands 32 rows per wave of the format's workgroup.
+// Matrix operands of the MFMA forward kernels, a process-wide setting (tgo_set_forward_operand):
+//   OPERAND_INT8    int8 quants on the int8 matrix instruction; every 32-value block result is scaled with two or
+//                   three fp32 vector operations (tgo_forward.hip), which bound those kernels.
+//   OPERAND_HALF    fp16 numbers holding the same integers exactly; one vector operation per result and block is
+//                   left (tgo_forward_half.hip).
+//   OPERAND_SCALED  both operands carry their scales: the dequantized q8_1 activation d * q and the dequantized
+//                   weight, each normalised by a power of two per row and rounded to fp16 once.  The matrix
+//                   instruction then accumulates the whole reduction and no vector instruction touches a result
+//                   before the epilogue (tgo_forward_scaled.hip): the only kind whose bound is the matrix pipe.
+//   OPERAND_AUTO    (default) the fastest kind measured per format.
+// `quant_type` 0 stands for a workspace that is quantized without knowing the format it will be used with
+// (tgo_quantize_q8_1 without a format): int8 unless another kind is forced.  The activation workspace is written for
+// one kind of operand and records which (Q8Workspace::tag); it must be consumed as that kind.
+enum ForwardOperand : int { OPERAND_INT8 = 0, OPERAND_HALF = 1, OPERAND_AUTO = 2, OPERAND_SCALED = 3 };
+int forward_operand_setting();
+void set_forward_operand_setting(int operand);
+// Formats of the scaled-operand kernel (all five).
+static constexpr bool scaled_forward_format(int quant_type) {
+    return quant_type == 11 || quant_type == 12 || quant_type == 13 || quant_type == 14 || quant_type == 22;
+}
+// The operand kind a call of this format uses under the current setting (never OPERAND_AUTO).
+static inline int forward_operand_kind(int quant_type) {
+    const int setting = forward_operand_setting();
+    if (setting == OPERAND_SCALED) {
+        return scaled_forward_format(quant_type) ? OPERAND_SCALED : quant_type == 22 ? OPERAND_HALF : OPERAND_INT8;
+    }
+    if (setting == OPERAND_AUTO) {
+        return quant_type == 22 ? OPERAND_HALF : OPERAND_INT8;
+    }
+    return setting;
+}
 // Waves per workgroup of the fp16-operand kernels, 32 activation rows each (8: the pipelined variant, measured 5 to
 // 11 % faster than the 4-wave one for the formats with 16-value scale groups, and no faster for the others).
 static constexpr int half_forward_waves(int quant_type) { return quant_type == 14 || quant_type == 22 ? 8 : 4; }
-static constexpr int forward_row_tile(int quant_type, bool half_operands) {
-    return half_operands ? 32 * half_forward_waves(quant_type) : (quant_type == 14 || quant_type == 22 ? 256 : 128);
-}
-// Matrix operands of the MFMA forward kernels: fp16 numbers holding the exact integers, or int8.  A process-wide
-// setting chooses one of them or (default) lets the format decide: IQ2_S (22), whose integer operand (2 s + 1) * m
-// needs 11 bits and therefore two int8 planes but a single fp16 number, runs a third faster with fp16 operands; the
-// formats whose operand fits a byte run 5 to 10 % faster with int8 (half the operand bytes through LDS and from the
-// workspace), and Q6_K (14) needs two numbers per value either way and runs the same.
-// `quant_type` 0 stands for a workspace that is quantized without knowing the format it will be used with
-// (tgo_quantize_q8_1 / tgo_mmq_forward_prepared): int8 unless fp16 is forced.  The activation workspace is written
-// for one kind of operand, so it must be consumed under the setting it was quantized with.
-enum ForwardOperand : int { OPERAND_INT8 = 0, OPERAND_HALF = 1, OPERAND_AUTO = 2 };
-int forward_operand_setting();
-void set_forward_operand_setting(int operand);
-static inline bool forward_half_operands(int quant_type) {
-    const int setting = forward_operand_setting();
-    return setting == OPERAND_AUTO ? quant_type == 22 : setting == OPERAND_HALF;
+// Row tile of one forward task; the task list is built for these.  int8 operands: 256 rows for the formats whose
+// weights unpack into two int8 planes (Q6_K = 14, IQ2_S = 22), 128 rows for the single-plane ones; exact fp16
+// operands: 32 rows per wave of the format's workgroup; scaled operands: 256 (four multiplying waves of 64 rows).
+static constexpr int forward_row_tile(int quant_type, int operand_kind) {
+    return operand_kind == OPERAND_SCALED ? 256
+           : operand_kind == OPERAND_HALF ? 32 * half_forward_waves(quant_type)
+                                          : (quant_type == 14 || quant_type == 22 ? 256 : 128);
 }
 constexpr int BACKWARD_ROW_TILE = 256;
 // Grad-input tasks of at most this many rows (a group's remainder) are listed behind the others and run by a
@@ -73,38 +91,56 @@ static inline bool use_gemv(int64_t rows, int64_t groups) {
     return groups <= 0 ? rows <= GEMV_DENSE_ROWS : rows <= 4 * groups;
 }
 
-// q8_1 workspace: quantized values, then fp32 scales, then fp32 sums, in one of three layouts over the same bytes.
-// The MFMA kernels want 32-row tiles in fragment order, as int8 or (half_tiles) as fp16 numbers holding the same
-// integers; the GEMV family reads a few rows along K, for which that order would scatter every 16 bytes into a
-// cache line of their own, so calls that take the GEMV family (use_gemv) quantize into plain int8 rows instead.
+// q8_1 workspace: quantized values, then fp32 scales, then fp32 sums, in one of four layouts over the same bytes.
+// The MFMA kernels want 32-row tiles in fragment order: int8, fp16 numbers holding the same integers, or (scaled)
+// the dequantized values d * q * 2^-e as fp16 with e chosen per row and super-block; the GEMV family reads a few
+// rows along K, for which that order would scatter every 16 bytes into a cache line of their own, so calls that
+// take the GEMV family (use_gemv) quantize into plain int8 rows instead.
+enum WorkspaceLayout : int { LAYOUT_INT8_TILES = 0, LAYOUT_HALF_TILES = 1, LAYOUT_ROWS = 2, LAYOUT_SCALED_TILES = 3 };
+constexpr uint32_t WORKSPACE_TAG_MAGIC = 0x71380000u;   // | layout: first word of the workspace's 1 KiB tail
+
 struct Q8Workspace {
-    int8_t * q;     // tiles: [rows_padded/32][K/32][2 halves][32 rows][16 bytes]   by_rows: [rows][K]
-                    // half_tiles: [rows_padded/32][K/32][2 k-halves][2 eighths x 32 rows][8 fp16]
-    float * d;      // tiles: [K/32][rows_padded]                                    by_rows: [rows][K/32]
+    int8_t * q;     // int8 tiles: [rows_padded/32][K/32][2 halves][32 rows][16 bytes]   rows: [rows][K]
+                    // half and scaled tiles: [rows_padded/32][K/32][2 k-halves][2 eighths x 32 rows][8 fp16]
+    float * d;      // tiles: [K/32][rows_padded]                                         rows: [rows][K/32]
     float * sum;    // same as d
+    float * power;  // scaled tiles: 2^E per row, [rows_padded]
+    uint16_t * block_sums;   // scaled tiles: fp16(sum * 2^-E) per block, [rows_padded/32][K/256][32 rows][8 blocks]
+    uint32_t * tag;          // WORKSPACE_TAG_MAGIC | layout, written by the quantizer
     int64_t rows_padded;
-    bool by_rows;
-    bool half_tiles;
+    int layout;
+    bool by_rows() const { return layout == LAYOUT_ROWS; }
+    bool half_tiles() const { return layout == LAYOUT_HALF_TILES; }
+    bool scaled_tiles() const { return layout == LAYOUT_SCALED_TILES; }
+    int operand_kind() const {
+        return layout == LAYOUT_SCALED_TILES ? OPERAND_SCALED : layout == LAYOUT_HALF_TILES ? OPERAND_HALF : OPERAND_INT8;
+    }
 };
 
 static inline int64_t pad_rows(int64_t rows) { return (rows + 31) / 32 * 32; }
 
-// (sized for the fp16 tiles whichever layout a call ends up using)
+// (sized for the scaled fp16 tiles whichever layout a call ends up using)
 static inline int64_t q8_workspace_bytes(int64_t rows, int64_t in_features) {
     const int64_t padded = pad_rows(rows);
     // the 1 KiB tail lets kernels fetch the scales of a whole 32-row tile with 16-byte loads even when the
-    // tile starts at the last row
-    return 2 * padded * in_features + 2 * padded * (in_features / 32) * static_cast<int64_t>(sizeof(float)) + 1024;
+    // tile starts at the last row; its first word is the layout tag
+    return 2 * padded * in_features + 2 * padded * (in_features / 32) * static_cast<int64_t>(sizeof(float)) +
+           padded * (in_features / 256) * (static_cast<int64_t>(sizeof(float)) + 16) + 1024;
 }
 
-static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t in_features, bool by_rows, int quant_type) {
+// `operand_kind`: OPERAND_INT8, OPERAND_HALF or OPERAND_SCALED (forward_operand_kind); ignored for by_rows.
+static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t in_features, bool by_rows, int operand_kind) {
     Q8Workspace view;
-    view.by_rows = by_rows;
-    view.half_tiles = !by_rows && forward_half_operands(quant_type);
+    view.layout = by_rows ? LAYOUT_ROWS
+                  : operand_kind == OPERAND_SCALED ? LAYOUT_SCALED_TILES
+                  : operand_kind == OPERAND_HALF ? LAYOUT_HALF_TILES : LAYOUT_INT8_TILES;
     view.rows_padded = pad_rows(rows);
     view.q = static_cast<int8_t *>(base);
     view.d = reinterpret_cast<float *>(view.q + 2 * view.rows_padded * in_features);
     view.sum = view.d + view.rows_padded * (in_features / 32);
+    view.power = view.sum + view.rows_padded * (in_features / 32);
+    view.block_sums = reinterpret_cast<uint16_t *>(view.power + view.rows_padded * (in_features / 256));
+    view.tag = reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(view.block_sums) + view.rows_padded * (in_features / 256) * 16);
     return view;
 }
 

@@ -86,12 +86,14 @@ EXPORTS = (
     "tgo_forward_operand",
 )
 
-OPERANDS = {"int8": 0, "half": 1, "auto": 2}
+OPERANDS = {"int8": 0, "half": 1, "auto": 2, "scaled": 3}
 
 
 def set_forward_operand(operand: str) -> None:
-    """Matrix operands of the MFMA forward kernels: "half" (fp16 numbers holding the exact integers), "int8", or
-    "auto" (the default: fp16 for IQ2_S, int8 otherwise)."""
+    """Matrix operands of the MFMA forward kernels: "int8", "half" (fp16 numbers holding the exact integers),
+    "scaled" (exact integer weights x the dequantized q8_1 activations as fp16, scaled once per super-block: the
+    kind bounded by the matrix pipe; Q6_K has no such kernel and keeps int8), or "auto" (the default: the
+    fastest kind measured per format)."""
     check(lib.tgo_set_forward_operand(OPERANDS[operand]))
 
 

@@ -278,13 +278,13 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
 }
 
 // LAYOUT_SCALED_TILES: the fp16 slabs of the half layout hold the dequantized values d * q instead of q, normalised
-// per row by the power of two 2^E that brings the row's largest magnitude into [2^8, 2^9), and rounded once to
-// fp16 (relative 2^-12); 2^E goes to the `power` plane, one number per row, and the block sums, scaled alike, to
-// `block_sums` as fp16, eight per row and super-block: the operand that meets the block minima of Q4_K/Q5_K.  The
-// scale and sum planes are written as in every layout.  The exponent needs the whole row, so a workgroup takes 32
-// rows x all of K: a first pass finds the rows' maxima, a second one quantizes chunk by chunk.  RESIDENT (K up to
-// 2048): the rows stay in registers between the passes; otherwise the second pass reads them again.
-template <bool RESIDENT>
+// per row and super-block (the 256 values of a row that a workgroup handles) by the power of two 2^e that brings the
+// super-block's largest block scale into [2^1, 2^2): every |d * q * 2^-e| stays below 2^9 and is rounded once to fp16
+// (relative 2^-12).  The block sums, scaled alike, go to `block_sums` as fp16, eight per row and super-block: the
+// operand that meets the block minima of Q4_K/Q5_K.  2^e goes to the `power` plane; a second, small pass
+// (scaled_row_power_kernel) turns it into 2^(e - E) with E the row's largest exponent, which the forward kernel
+// multiplies into the fragments of the super-block (exact: a power of two), and writes 2^E per row.  The scale and
+// sum planes are written as in every layout.
 __global__ __launch_bounds__(256) void quantize_q8_1_scaled_kernel(const uint16_t * __restrict__ input,
                                                                   int8_t * __restrict__ q_out,
                                                                   float * __restrict__ d_out,
@@ -301,15 +301,16 @@ __global__ __launch_bounds__(256) void quantize_q8_1_scaled_kernel(const uint16_
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         *tag = WORKSPACE_TAG_MAGIC | LAYOUT_SCALED_TILES;
     }
-    constexpr int GROUP = 8;   // chunks of 256 values whose loads are in flight together
+    // (workgroup order as in quantize_q8_1_kernel: neighbouring workgroups take neighbouring chunks of the same rows)
     const int chunks = in_features / 256;
     const int64_t rows_padded = (static_cast<int64_t>(rows) + 31) / 32 * 32;
     __shared__ __attribute__((aligned(16))) uint8_t tile[16 * 1024];
-    __shared__ __attribute__((aligned(16))) float scales[2][8][32];   // d and sum of the chunk: [which][block][row]
-    __shared__ __attribute__((aligned(16))) uint16_t sums_half[32][8];
+    __shared__ __attribute__((aligned(16))) float scales[2][8][32];   // d and sum of the tile: [which][block][row]
     __shared__ __attribute__((aligned(16))) float powers[32];
+    __shared__ __attribute__((aligned(16))) uint16_t sums_half[32][8];
     const int tid = threadIdx.x;
-    const int row_tile = blockIdx.x;
+    const int row_tile = blockIdx.x / chunks;                 // 32-row tile
+    const int chunk = blockIdx.x - row_tile * chunks;         // 256-value column chunk
     const int blocks_per_row = in_features / 32;
     const int lane_k = tid & 31;       // 8 values each
     const int block = lane_k >> 2;     // 32-value block inside the chunk
@@ -325,125 +326,96 @@ __global__ __launch_bounds__(256) void quantize_q8_1_scaled_kernel(const uint16_
         source[pass] = min(row, last_row);
         if (gather != nullptr) {   // uniform
             source[pass] = gather[source[pass]];
+        }
+    }
+    uint4 bits[4];
+#pragma unroll
+    for (int pass = 0; pass < 4; ++pass) {
+        if (gather != nullptr) {
             present[pass] = present[pass] && source[pass] >= 0 && source[pass] < input_rows;
             source[pass] = present[pass] ? source[pass] : 0;
         }
+        bits[pass] = *reinterpret_cast<const uint4 *>(input + source[pass] * in_features + chunk * 256 + lane_k * 8);
     }
-    auto load_chunk = [&](int chunk, uint4 (&bits)[4]) {
-        const int clamped = min(chunk, chunks - 1);
-#pragma unroll
-        for (int pass = 0; pass < 4; ++pass) {
-            bits[pass] = *reinterpret_cast<const uint4 *>(input + source[pass] * in_features + clamped * 256 + lane_k * 8);
-            if (!present[pass] || chunk >= chunks) {
-                bits[pass] = uint4{0, 0, 0, 0};
-            }
-        }
-    };
-    // ---- first pass: the largest magnitude of each of the thread's four rows
-    uint4 resident[RESIDENT ? GROUP : 1][4];
-    float largest[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-    for (int first = 0; first < chunks; first += GROUP) {
-        uint4 group[GROUP][4];
-#pragma unroll
-        for (int c = 0; c < GROUP; ++c) {
-            load_chunk(first + c, group[c]);
-        }
-#pragma unroll
-        for (int c = 0; c < GROUP; ++c) {
-#pragma unroll
-            for (int pass = 0; pass < 4; ++pass) {
-                float x[8];
-                unpack_bf16x8(group[c][pass], x);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    largest[pass] = fmaxf(largest[pass], fabsf(x[i]));
-                }
-                if constexpr (RESIDENT) {
-                    resident[c][pass] = group[c][pass];
-                }
-            }
-        }
-    }
-    float inverse[4];
 #pragma unroll
     for (int pass = 0; pass < 4; ++pass) {
-        float amax = largest[pass];
+        const int rr = (tid >> 5) + 8 * pass;
+        float x[8];
+        const uint4 row_bits = present[pass] ? bits[pass] : uint4{0, 0, 0, 0};
+        unpack_bf16x8(row_bits, x);
+        uint32_t packed[2], halves[4];
+        int magnitude[8];
+        float d, total;
+        quantize_eight(row_bits, x, packed, d, total, halves, magnitude);
+        // the row's 32 lanes hold its eight block scales; the largest one fixes the super-block's exponent
+        float largest = fmaxf(d, __shfl_xor(d, 4));
+        largest = fmaxf(largest, __shfl_xor(largest, 8));
+        largest = fmaxf(largest, __shfl_xor(largest, 16));
+        int exponent = static_cast<int>(__float_as_uint(largest) >> 23);   // biased; d is never negative
+        exponent = min(max(exponent, 2), 254);
+        const float power = __uint_as_float(static_cast<uint32_t>(exponent - 1) << 23);     // 2^e
+        const float inverse = __uint_as_float(static_cast<uint32_t>(255 - exponent) << 23);   // 2^-e
+        const float lane_scale = d * inverse;
+        const uint32_t words[4] = {row_bits.x, row_bits.y, row_bits.z, row_bits.w};
 #pragma unroll
-        for (int offset = 1; offset < 32; offset <<= 1) {
-            amax = fmaxf(amax, __shfl_xor(amax, offset));
+        for (int pair = 0; pair < 4; ++pair) {
+            const half2_t values = {static_cast<_Float16>(static_cast<float>(magnitude[2 * pair]) * lane_scale),
+                                    static_cast<_Float16>(static_cast<float>(magnitude[2 * pair + 1]) * lane_scale)};
+            halves[pair] = __builtin_bit_cast(uint32_t, values) | (words[pair] & 0x80008000u);
         }
-        int exponent = static_cast<int>(__float_as_uint(amax) >> 23);   // biased
-        exponent = min(max(exponent, 9), 254);
-        inverse[pass] = __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-E
+        // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
+        *reinterpret_cast<uint4 *>(tile + block * 2048 + (quarter >> 1) * 1024 + (rr + 32 * (quarter & 1)) * 16) =
+            make_uint4(halves[0], halves[1], halves[2], halves[3]);
+        if (quarter == 0) {
+            scales[0][block][rr] = d;
+            scales[1][block][rr] = total;
+            sums_half[rr][block] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(total * inverse));
+        }
         if (lane_k == 0) {
-            powers[(tid >> 5) + 8 * pass] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^E
+            powers[rr] = power;
         }
     }
     __syncthreads();
-    if (tid < 8) {
-        *reinterpret_cast<float4 *>(power_out + row_tile * 32 + tid * 4) = *reinterpret_cast<const float4 *>(&powers[tid * 4]);
+    // the 32 rows of a block are one 128-byte line of each scale plane: 2 planes x 8 blocks x 8 pieces
+    if (tid < 128) {
+        const int which = tid >> 6, b = (tid >> 3) & 7, piece = tid & 7;
+        float * plane = which == 0 ? d_out : sum_out;
+        *reinterpret_cast<float4 *>(plane + static_cast<int64_t>(chunk * 8 + b) * rows_padded + row_tile * 32 + piece * 4) =
+            *reinterpret_cast<const float4 *>(&scales[which][b][piece * 4]);
+    } else if (tid < 136) {
+        const int piece = tid - 128;
+        *reinterpret_cast<float4 *>(power_out + static_cast<int64_t>(chunk) * rows_padded + row_tile * 32 + piece * 4) =
+            *reinterpret_cast<const float4 *>(&powers[piece * 4]);
+    } else if (tid >= 192 && tid < 224) {
+        const int row = tid - 192;
+        *reinterpret_cast<uint4 *>(block_sums_out + ((static_cast<int64_t>(row_tile) * chunks + chunk) * 32 + row) * 8) =
+            *reinterpret_cast<const uint4 *>(&sums_half[row][0]);
     }
-    // ---- second pass: quantize, chunk by chunk
-    auto quantize_chunk = [&](int chunk, const uint4 (&bits)[4]) {
+    uint4 * dst = reinterpret_cast<uint4 *>(q_out + (static_cast<int64_t>(row_tile) * blocks_per_row + chunk * 8) * 2048);
+    const uint4 * src = reinterpret_cast<const uint4 *>(tile);
 #pragma unroll
-        for (int pass = 0; pass < 4; ++pass) {
-            const int rr = (tid >> 5) + 8 * pass;
-            float x[8];
-            unpack_bf16x8(bits[pass], x);
-            uint32_t packed[2], halves[4];
-            int magnitude[8];
-            float d, total;
-            quantize_eight(bits[pass], x, packed, d, total, halves, magnitude);
-            const float lane_scale = d * inverse[pass];
-            const uint32_t words[4] = {bits[pass].x, bits[pass].y, bits[pass].z, bits[pass].w};
-#pragma unroll
-            for (int pair = 0; pair < 4; ++pair) {
-                const half2_t values = {static_cast<_Float16>(static_cast<float>(magnitude[2 * pair]) * lane_scale),
-                                        static_cast<_Float16>(static_cast<float>(magnitude[2 * pair + 1]) * lane_scale)};
-                halves[pair] = __builtin_bit_cast(uint32_t, values) | (words[pair] & 0x80008000u);
-            }
-            // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
-            *reinterpret_cast<uint4 *>(tile + block * 2048 + (quarter >> 1) * 1024 + (rr + 32 * (quarter & 1)) * 16) =
-                make_uint4(halves[0], halves[1], halves[2], halves[3]);
-            if (quarter == 0) {
-                scales[0][block][rr] = d;
-                scales[1][block][rr] = total;
-                sums_half[rr][block] = __builtin_bit_cast(uint16_t, static_cast<_Float16>(total * inverse[pass]));
-            }
-        }
-        __syncthreads();
-        if (tid < 128) {
-            const int which = tid >> 6, b = (tid >> 3) & 7, piece = tid & 7;
-            float * plane = which == 0 ? d_out : sum_out;
-            *reinterpret_cast<float4 *>(plane + static_cast<int64_t>(chunk * 8 + b) * rows_padded + row_tile * 32 + piece * 4) =
-                *reinterpret_cast<const float4 *>(&scales[which][b][piece * 4]);
-        } else if (tid >= 192 && tid < 224) {
-            const int row = tid - 192;
-            *reinterpret_cast<uint4 *>(block_sums_out + ((static_cast<int64_t>(row_tile) * chunks + chunk) * 32 + row) * 8) =
-                *reinterpret_cast<const uint4 *>(&sums_half[row][0]);
-        }
-        uint4 * dst = reinterpret_cast<uint4 *>(q_out + (static_cast<int64_t>(row_tile) * blocks_per_row + chunk * 8) * 2048);
-        const uint4 * src = reinterpret_cast<const uint4 *>(tile);
-#pragma unroll
-        for (int piece = 0; piece < 4; ++piece) {
-            dst[tid + 256 * piece] = src[tid + 256 * piece];
-        }
-        __syncthreads();
-    };
-    if constexpr (RESIDENT) {
-#pragma unroll
-        for (int c = 0; c < GROUP; ++c) {
-            if (c < chunks) {   // uniform
-                quantize_chunk(c, resident[c]);
-            }
-        }
-    } else {
-        for (int c = 0; c < chunks; ++c) {
-            uint4 bits[4];
-            load_chunk(c, bits);
-            quantize_chunk(c, bits);
-        }
+    for (int piece = 0; piece < 4; ++piece) {
+        dst[tid + 256 * piece] = src[tid + 256 * piece];
     }
+}
+
+// Second pass of the scaled layout: power[sb][row] = 2^e  ->  2^(e - E), row_power[row] = 2^E with E = max over sb.
+__global__ __launch_bounds__(256) void scaled_row_power_kernel(float * __restrict__ power, float * __restrict__ row_power,
+                                                              int64_t rows_padded, int chunks) {
+    const int64_t row = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    if (row >= rows_padded) {
+        return;
+    }
+    float largest = 0.0f;
+    for (int c = 0; c < chunks; ++c) {
+        largest = fmaxf(largest, power[c * rows_padded + row]);
+    }
+    // (all entries are powers of two between 2^-126 and 2^126: the quotient is exact)
+    const float inverse = __uint_as_float((254u - (__float_as_uint(largest) >> 23)) << 23);
+    for (int c = 0; c < chunks; ++c) {
+        power[c * rows_padded + row] *= inverse;
+    }
+    row_power[row] = largest;
 }
 
 hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, int64_t rows,
@@ -458,22 +430,18 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
         return hipGetLastError();
     }
     const int r = static_cast<int>(rows), k = static_cast<int>(in_features);
-    if (ws.scaled_tiles()) {
-        const dim3 grid(static_cast<unsigned>(ws.rows_padded / 32));
-        if (in_features <= 2048) {
-            quantize_q8_1_scaled_kernel<true><<<grid, 256, 0, stream>>>(
-                input, ws.q, ws.d, ws.sum, ws.power, ws.block_sums, ws.tag, r, k, gather, input_rows, on_the_side);
-        } else {
-            quantize_q8_1_scaled_kernel<false><<<grid, 256, 0, stream>>>(
-                input, ws.q, ws.d, ws.sum, ws.power, ws.block_sums, ws.tag, r, k, gather, input_rows, on_the_side);
-        }
-        return hipGetLastError();
-    }
     const int64_t workgroups = ws.rows_padded / 32 * (in_features / 256);
     if (workgroups > 0x7fffffffLL) {
         return hipErrorInvalidValue;
     }
     const dim3 grid(static_cast<unsigned>(workgroups));
+    if (ws.scaled_tiles()) {
+        quantize_q8_1_scaled_kernel<<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, ws.power, ws.block_sums, ws.tag, r, k,
+                                                              gather, input_rows, on_the_side);
+        scaled_row_power_kernel<<<static_cast<unsigned>((ws.rows_padded + 255) / 256), 256, 0, stream>>>(
+            ws.power, ws.row_power, ws.rows_padded, k / 256);
+        return hipGetLastError();
+    }
     if (ws.half_tiles()) {
         quantize_q8_1_kernel<LAYOUT_HALF_TILES><<<grid, 256, 0, stream>>>(input, ws.q, ws.d, ws.sum, ws.tag, r, k, gather,
                                                                            input_rows, on_the_side);
@@ -486,12 +454,13 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
 
 // Workspace inspection for tests: the quants, scales and sums as plain rows, whichever layout the quantizer wrote
 // (read from the workspace's tag; a workspace without a valid tag yields zeros).  The scaled layout stores d * q:
-// its quants are recovered as round(value * 2^E / d), exact because the fp16 rounding moves a value by less than
+// its quants are recovered as round(value * 2^e / d), exact because the fp16 rounding moves a value by less than
 // 127 * 2^-12 of a quant step (values that the normalisation pushed below the fp16 range come back as zero).
 __global__ __launch_bounds__(256) void q8_unpack_kernel(const int8_t * __restrict__ q_frag,
                                                        const float * __restrict__ d_in,
                                                        const float * __restrict__ sum_in,
                                                        const float * __restrict__ power_in,
+                                                       const float * __restrict__ row_power_in,
                                                        const uint32_t * __restrict__ tag,
                                                        int8_t * __restrict__ q, float * __restrict__ d,
                                                        float * __restrict__ sum, int rows,
@@ -535,7 +504,7 @@ __global__ __launch_bounds__(256) void q8_unpack_kernel(const int8_t * __restric
             values[(static_cast<int64_t>(row >> 5) * blocks_per_row + block) * 1024 + half * 512 +
                    ((row & 31) + 32 * (byte >> 3)) * 8 + (byte & 7)]);
         if (layout == LAYOUT_SCALED_TILES) {
-            value = scale == 0.0f ? 0.0f : rintf(value * power_in[row] / scale);
+            value = scale == 0.0f ? 0.0f : rintf(value * (power_in[(k >> 8) * rows_padded + row] * row_power_in[row]) / scale);
         }
         q[index] = static_cast<int8_t>(value);
     }
@@ -549,7 +518,7 @@ hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float
                             int64_t in_features, hipStream_t stream) {
     const int64_t total = rows * in_features;
     q8_unpack_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(
-        ws.q, ws.d, ws.sum, ws.power, ws.tag, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features));
+        ws.q, ws.d, ws.sum, ws.power, ws.row_power, ws.tag, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features));
     return hipGetLastError();
 }
 

@@ -604,6 +604,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     args.dx = ws.d;
     args.sx = ws.sum;
     args.power = ws.power;
+    args.row_power = ws.row_power;
     args.block_sums = ws.block_sums;
     args.y = output;
     args.rows = rows;

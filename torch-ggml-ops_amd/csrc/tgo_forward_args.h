@@ -19,7 +19,8 @@ struct ForwardArgs {
     const int8_t * qx;               // int8 tiles, or fp16 tiles (Q8Workspace::layout)
     const float * dx;
     const float * sx;
-    const float * power;             // scaled tiles only: 2^e per row and super-block
+    const float * power;             // scaled tiles only: 2^(e - E) per row and super-block
+    const float * row_power;         // scaled tiles only: 2^E per row
     const uint16_t * block_sums;     // scaled tiles only: fp16 block sums, eight per row and super-block
     uint16_t * y;
     uint16_t * y_second;
@@ -41,14 +42,15 @@ struct ForwardArgs {
 };
 
 // The (column tile, projection, task) of this workgroup; false when the slot holds no task.
-TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second, int & expert, int & row_start,
-                             int & row_end) {
+// `linear`: position in the launch order of workgroups (blockIdx.x for kernels that run one task per workgroup).
+TGO_DEVICE bool forward_pick_linear(const ForwardArgs & a, int linear, int & n_tile, bool & second, int & expert,
+                                    int & row_start, int & row_end) {
     int task;
     const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + a.dense_row_tile - 1) / a.dense_row_tile;
     if (a.task_count != nullptr) {
-        xcd_chunk(blockIdx.x, a.n_tiles * a.projections, tasks, min(a.task_early[0], tasks), n_tile, task);
+        xcd_chunk(linear, a.n_tiles * a.projections, tasks, min(a.task_early[0], tasks), n_tile, task);
     } else {
-        xcd_tile<FWD_XCD_RUN>(blockIdx.x, a.n_tiles * a.projections, tasks, n_tile, task);
+        xcd_tile<FWD_XCD_RUN>(linear, a.n_tiles * a.projections, tasks, n_tile, task);
     }
     second = n_tile >= a.n_tiles;
     n_tile -= second ? a.n_tiles : 0;
@@ -68,6 +70,11 @@ TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second,
         row_end = min(a.rows, row_start + a.dense_row_tile);
     }
     return true;
+}
+
+TGO_DEVICE bool forward_pick(const ForwardArgs & a, int & n_tile, bool & second, int & expert, int & row_start,
+                             int & row_end) {
+    return forward_pick_linear(a, blockIdx.x, n_tile, second, expert, row_start, row_end);
 }
 
 // Launch of the fp16-operand kernels for arguments prepared by the common launcher (tgo_forward.hip).

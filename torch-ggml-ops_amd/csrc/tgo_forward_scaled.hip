@@ -2,12 +2,14 @@
 // task, bounded by the matrix pipe instead of the vector pipe.
 //
 //   y[r, n] = 2^(E[r] + S[n]) * sum over k of  w[n, k] * h[r, k]      (v_mfma_f32_32x32x16_f16, fp32 accumulation)
-//   h[r, k] = fp16(dx * qx * 2^-E[r])     the dequantized q8_1 activation, normalised per row, rounded once
+//   h[r, k] = fp16(dx * qx * 2^-e[r, s]) * 2^(e[r, s] - E[r])   the dequantized q8_1 activation, rounded once after a
+//             normalisation per row and super-block s, then brought to the row's common exponent (exact)
 //   w[n, k] = fp16(v[n, k] * fp16(scale * 2^-S[n]))   the integer operand v = sub-scale x quant (exact in fp16) times
 //             the weight scale of its group, normalised per weight row
 // Q4_K/Q5_K: v = q, scale = d * sc, and the minimum term -dmin * m * (block sum) is one more reduction step per
-// super-block whose operands are fp16(-dmin * m * 2^-S[n]) and fp16(block sum * 2^-E[r]).  The quantizer writes h, the
-// block sums and 2^E (quantize_q8_1_scaled_kernel); S[n] comes from a scan of the weight row's super-block scales.
+// super-block whose operands are fp16(-dmin * m * 2^-S[n]) and the block sum treated like h.  The quantizer writes
+// the normalised values and block sums, 2^(e - E) and 2^E (quantize_q8_1_scaled_kernel, scaled_row_power_kernel);
+// S[n] comes from a scan of the weight row's super-block scales.
 // The algebra is the q8_1 one (same quants, block scales and sums as the int8 kernels of tgo_forward.hip); what
 // differs is that both operands carry their scales into the matrix instruction, each rounded to fp16 once (relative
 // 2^-11: the reference keeps its own scale products d * sc and dmin * m as halves too,
@@ -24,6 +26,12 @@
 // wave that feeds the matrix pipe and one that keeps the vector pipe busy.  A super-block is two stages of 128
 // values; the operand tile of a stage (32 KiB, fragment order) is double buffered and one barrier per stage hands
 // it over: while the multipliers work on stage g, the unpackers write stage g + 1.
+//
+// A workgroup is persistent: it owns every gridDim.x-th (task, column tile) item of the launch and runs their
+// super-blocks as one stream, so an item's first loads (task description, packed blocks, the scan of its scales,
+// activation fragments) are requested while the item before it is still being multiplied, and its results are
+// stored while the unpackers already work on the next one.  With one item per workgroup those latencies and the
+// epilogue, none of them overlapped by anything on a CU that holds a single workgroup, were 40 % of the kernel's time.
 #include <type_traits>
 
 #include "tgo_device.h"
@@ -52,6 +60,14 @@ static_assert(FSC_ROWS == forward_row_tile(12, OPERAND_SCALED), "task rows match
 #define FSC_X_AHEAD 8
 #endif
 
+constexpr int FSC_MAX_ITEMS = 64;      // items per workgroup (one wave builds the table)
+constexpr int FSC_GRID = 256;          // one workgroup per CU
+constexpr int FSC_STAGE_PITCH = 68;    // bf16 per staged row: 64 columns + padding (34 words: 32 rows on 32 different banks)
+
+struct ScaledItem {
+    int expert, row_start, row_end, tile;   // tile: column tile + n_tiles * projection
+};
+
 template <int TYPE>
 struct ScaledLds {
     static constexpr bool K45 = TYPE == Q4_K || TYPE == Q5_K;
@@ -63,7 +79,10 @@ struct ScaledLds {
     alignas(16) uint8_t wq[2][FSC_TILE_BYTES];                 // operand tiles of two stages
     alignas(16) uint8_t raw[4][2][32 * RAW_SLOT];              // per unpacking wave: packed blocks of two super-blocks
     alignas(16) uint8_t mins[2][K45 ? FWD_NT * 512 : 16];      // fp16(-dmin * m * 2^-S): [tile][32 rows][8 blocks], by parity
-    alignas(16) float row_power[FWD_TN];                       // 2^S of the tile's weight rows
+    alignas(16) float row_power[2][FWD_TN];                    // 2^S of the tile's weight rows, by the item's parity
+    alignas(16) uint16_t staging[4][32 * FSC_STAGE_PITCH];     // per multiplying wave: 32 rows x 64 columns of results
+    ScaledItem items[FSC_MAX_ITEMS];
+    int item_count;
     std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;
 };
 
@@ -103,59 +122,113 @@ constexpr int scale_offset() { return TYPE == Q3_K ? 108 : TYPE == Q6_K ? 208 : 
 __device__ unsigned long long fsc_times[8][2][96];
 // phase accumulators in scalar registers; nothing is stored before the end of the kernel
 #define FSC_LAP(slot) do { const unsigned long long now_ = __builtin_readcyclecounter(); lap[slot] += now_ - lap_last; lap_last = now_; } while (0)
+#define FSC_LAP_DUMP(role) do { if (profiled >= 0 && lane == 0) { for (int i_ = 0; i_ < 10; ++i_) fsc_times[profiled][role][i_ + 1] = lap[i_]; fsc_times[profiled][role][90] = n_items; fsc_times[profiled][role][94] = wall_clock64() - wall_start; } } while (0)
 #else
 #define FSC_LAP(slot) do {} while (0)
+#define FSC_LAP_DUMP(role) do {} while (0)
 #endif
 
+// Stores a 32-row x 64-column block of results that the matrix instructions left transposed (weights as the A
+// operand: the lane holds row l32 and, as element v of tile t, column 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4) as
+// bf16 rows: the wave transposes through `stage` (32 x FSC_STAGE_PITCH bf16 that only this wave touches) and every
+// lane stores 16-byte pieces, whole 128-byte rows.  `dst` points at row 0, column 0; rows >= valid_rows and columns >=
+// valid_cols are skipped.  The 16-byte path needs row_stride % 8 == 0 (dst is then 16-byte aligned: the tensor is,
+// and column tiles start at multiples of 64).
+TGO_DEVICE void store_rows_32x64(uint16_t * stage, const v16f (&tiles)[2], uint16_t * dst, int64_t row_stride,
+                                 int valid_rows, int valid_cols, int lane) {
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            *reinterpret_cast<uint2 *>(&stage[l32 * FSC_STAGE_PITCH + t * 32 + 8 * j + 4 * half]) =
+                make_uint2(pack_bf16x2(tiles[t][4 * j], tiles[t][4 * j + 1]), pack_bf16x2(tiles[t][4 * j + 2], tiles[t][4 * j + 3]));
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    const bool wide = (row_stride & 7) == 0;
+#pragma unroll
+    for (int p = 0; p < 4; ++p) {
+        const int id = lane + 64 * p;
+        const int r = id >> 3;
+        const int c = (id & 7) * 8;
+        if (r < valid_rows && c < valid_cols) {
+            const uint16_t * values = &stage[r * FSC_STAGE_PITCH + c];
+            if (wide && c + 8 <= valid_cols) {
+                // (rows of the staging area start 8-byte aligned: two 8-byte reads)
+                const uint2 low = *reinterpret_cast<const uint2 *>(values);
+                const uint2 high = *reinterpret_cast<const uint2 *>(values + 4);
+                *reinterpret_cast<uint4 *>(dst + r * row_stride + c) = make_uint4(low.x, low.y, high.x, high.y);
+            } else {
+                for (int e = 0; e < 8 && c + e < valid_cols; ++e) {
+                    dst[r * row_stride + c + e] = values[e];
+                }
+            }
+        }
+    }
+    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+}
+
 template <int TYPE, bool WIDE>
-__global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(const ForwardArgs a) {
-#ifdef FSC_TIMING
-    const int profiled_early = blockIdx.x % 1000 == 7 && blockIdx.x / 1000 < 8 ? blockIdx.x / 1000 : -1;
-    if (profiled_early >= 0 && threadIdx.x == 0) fsc_times[profiled_early][0][0] = __builtin_readcyclecounter();
-    if (profiled_early >= 0 && threadIdx.x == 0) fsc_times[profiled_early][0][93] = wall_clock64();
-    if (profiled_early >= 0 && threadIdx.x == 256) fsc_times[profiled_early][1][0] = __builtin_readcyclecounter();
-#endif
+__global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(const ForwardArgs a, const int total_slots) {
     using F = Format<TYPE>;
     using L = ScaledLds<TYPE>;
     constexpr bool K45 = L::K45;
     __shared__ L lds;
 
-    int n_tile, expert, row_start, row_end;
-    bool second;
-    if (!forward_pick(a, n_tile, second, expert, row_start, row_end)) {
-        return;
-    }
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int l32 = lane & 31;
     const int half = lane >> 5;
-#ifdef FSC_TIMING
-    const int profiled = (wave == 0 || wave == 4) ? profiled_early : -1;
-    if (profiled >= 0 && tid == 0) { fsc_times[profiled][0][95] = (static_cast<unsigned long long>(row_end - row_start) << 32) | static_cast<unsigned>(n_tile); }
-    unsigned long long lap[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-    unsigned long long lap_last = __builtin_readcyclecounter();
-    if (profiled >= 0 && lane == 0) { fsc_times[profiled][wave >> 2][90] = lap_last; }
-#endif
 
-    const uint8_t * weights = (second ? a.packed_second : a.packed) + static_cast<int64_t>(expert) * a.bytes_per_expert;
-    uint16_t * const y = second ? a.y_second : a.y;
-    const int n0 = n_tile * FWD_TN;
-    const int super_blocks = a.in_features / QK_K;
-    const int tile_rows = min(FWD_TN, a.out_features - n0);   // weight rows of this tile that exist
-
+    // item table: slot i of this workgroup is position blockIdx.x + i * gridDim.x of the launch order (gridDim.x is
+    // a multiple of the XCD count, so all of them map to this workgroup's XCD); empty slots are squeezed out
+    if (wave == 0) {
+        ScaledItem item = {0, 0, 0, -1};
+        const int64_t linear = blockIdx.x + static_cast<int64_t>(lane) * gridDim.x;
+        if (linear < total_slots) {
+            int n_tile, expert, row_start, row_end;
+            bool second;
+            if (forward_pick_linear(a, static_cast<int>(linear), n_tile, second, expert, row_start, row_end)) {
+                item = ScaledItem{expert, row_start, row_end, n_tile + (second ? a.n_tiles : 0)};
+            }
+        }
+        const bool valid = item.tile >= 0;
+        const unsigned long long mask = __ballot(valid);
+        if (valid) {
+            lds.items[__popcll(mask & ((1ull << lane) - 1ull))] = item;
+        }
+        if (lane == 0) {
+            lds.item_count = __popcll(mask);
+        }
+    }
     if constexpr (TYPE == IQ2_S) {
         expand_iq2s_selectors(lds.codebook, tid, FSC_THREADS);
-        __syncthreads();
     }
+    __syncthreads();
+    const int n_items = lds.item_count;
+    if (n_items == 0) {
+        return;
+    }
+#ifdef FSC_TIMING
+    const int profiled = (wave == 0 || wave == 4) && blockIdx.x % 32 == 5 ? blockIdx.x / 32 : -1;
+    unsigned long long lap[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    unsigned long long lap_last = __builtin_readcyclecounter();
+    const unsigned long long wall_start = wall_clock64();
+#endif
+    const int super_blocks = a.in_features / QK_K;
+    const int total = n_items * super_blocks;   // super-blocks of this workgroup's stream
+    auto item_field = [&](int item, int field) {
+        return __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(&lds.items[item])[field]);
+    };
 
     if (wave >= 4) {
         // ---------------- unpacking wave ----------------
         const int dw = wave - 4;
-        // rows past the end of the weight matrix repeat its last row (their results are never stored)
-        const int first_row = min(32 * dw, tile_rows - 1);
-        const int rows_valid = max(1, min(32, tile_rows - 32 * dw));
-        const uint8_t * const wave_weights = weights + static_cast<int64_t>(n0 + first_row) * a.row_bytes;
         constexpr int RAW_UNITS = K45 ? F::BLOCK_BYTES / 16 : 1;
         constexpr int RAW_REGS = K45 ? (32 * RAW_UNITS + 63) / 64 : 1;
         using W = WideStage<TYPE>;
@@ -163,27 +236,83 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         constexpr int SLOT_PITCH = K45 ? F::BLOCK_BYTES : (WIDE ? W::PITCH : F::RAW_PITCH);
         constexpr int SLOT_FRONT = K45 ? 0 : (WIDE ? W::FRONT : F::RAW_SHIFT);
 
-        // ---- S of this lane's weight row: the largest weight magnitude over the row's super-blocks goes to [2^8, 2^9)
-        const uint8_t * const lane_row_blocks = wave_weights + static_cast<int64_t>(min(l32, rows_valid - 1)) * a.row_bytes;
-        float reach = 0.0f;
-        for (int kb = half; kb < super_blocks; kb += 2) {
-            const uint8_t * blk = lane_row_blocks + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
-            if constexpr (K45) {
-                const uint32_t pair = *reinterpret_cast<const uint32_t *>(blk);
-                reach = fmaxf(reach, fabsf(half_bits_to_float(pair & 0xffffu)) * weight_reach<TYPE>());
-                reach = fmaxf(reach, fabsf(half_bits_to_float(pair >> 16)) * 63.0f);
-            } else {
-                const uint32_t bits = *reinterpret_cast<const uint16_t *>(blk + scale_offset<TYPE>());
-                reach = fmaxf(reach, fabsf(half_bits_to_float(bits)) * weight_reach<TYPE>());
+        // Position of one stage of this wave's pipeline in the stream, with what it needs to know about the item:
+        // the wave's 32 weight rows (rows past the end of the weight matrix repeat its last row; their results are
+        // never stored).  A cursor at the last super-block stays there: stages that look past the end repeat it.
+        struct Cursor {
+            int item, kb;
+            const uint8_t * weights;   // of the item's expert and projection
+            const uint8_t * rows;      // first of the wave's weight rows
+            int n0, rows_valid;
+        };
+        auto open_item = [&](Cursor & c, int item) {
+            c.item = item;
+            c.kb = 0;
+            const int tile = item_field(item, 3);
+            const bool second = tile >= a.n_tiles;
+            c.weights = (second ? a.packed_second : a.packed) + static_cast<int64_t>(item_field(item, 0)) * a.bytes_per_expert;
+            c.n0 = (second ? tile - a.n_tiles : tile) * FWD_TN;
+            const int tile_rows = min(FWD_TN, a.out_features - c.n0);
+            c.rows_valid = max(1, min(32, tile_rows - 32 * dw));
+            c.rows = c.weights + static_cast<int64_t>(c.n0 + min(32 * dw, tile_rows - 1)) * a.row_bytes;
+        };
+        auto step = [&](Cursor & c) {
+            if (c.kb + 1 < super_blocks) {
+                ++c.kb;
+            } else if (c.item + 1 < n_items) {
+                open_item(c, c.item + 1);
             }
-        }
-        reach = fmaxf(reach, __shfl_xor(reach, 32));
-        int reach_exponent = static_cast<int>(__float_as_uint(reach) >> 23);   // biased
-        reach_exponent = min(max(reach_exponent, 9), 254);
-        const float shrink = __uint_as_float(static_cast<uint32_t>(262 - reach_exponent) << 23);   // 2^-S
-        if (half == 0) {
-            lds.row_power[32 * dw + l32] = __uint_as_float(static_cast<uint32_t>(reach_exponent - 8) << 23);   // 2^S
-        }
+        };
+
+        // ---- S of this lane's weight row: the largest weight magnitude over the row's super-blocks goes to
+        // [2^8, 2^9).  The scale words of the first eight super-blocks are requested an item ahead.
+        constexpr int SCAN_REGS = 4;
+        auto scan_request = [&](const Cursor & c, uint32_t (&words)[SCAN_REGS]) {
+            const uint8_t * blocks = c.rows + static_cast<int64_t>(min(l32, c.rows_valid - 1)) * a.row_bytes;
+#pragma unroll
+            for (int i = 0; i < SCAN_REGS; ++i) {
+                const int kb = min(half + 2 * i, super_blocks - 1);
+                const uint8_t * blk = blocks + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+                if constexpr (K45) {
+                    words[i] = *reinterpret_cast<const uint32_t *>(blk);
+                } else {
+                    words[i] = *reinterpret_cast<const uint16_t *>(blk + scale_offset<TYPE>());
+                }
+            }
+        };
+        auto scan_word = [&](uint32_t word) {
+            float reach = fabsf(half_bits_to_float(word & 0xffffu)) * weight_reach<TYPE>();
+            if constexpr (K45) {
+                reach = fmaxf(reach, fabsf(half_bits_to_float(word >> 16)) * 63.0f);
+            }
+            return reach;
+        };
+        // returns 2^-S and leaves 2^S for the multiplying waves
+        auto scan_finish = [&](const Cursor & c, const uint32_t (&words)[SCAN_REGS]) {
+            float reach = 0.0f;
+#pragma unroll
+            for (int i = 0; i < SCAN_REGS; ++i) {
+                reach = fmaxf(reach, scan_word(words[i]));
+            }
+            if (super_blocks > 2 * SCAN_REGS) {   // long rows: the rest, read here
+                const uint8_t * blocks = c.rows + static_cast<int64_t>(min(l32, c.rows_valid - 1)) * a.row_bytes;
+                for (int kb = 2 * SCAN_REGS + half; kb < super_blocks; kb += 2) {
+                    const uint8_t * blk = blocks + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+                    if constexpr (K45) {
+                        reach = fmaxf(reach, scan_word(*reinterpret_cast<const uint32_t *>(blk)));
+                    } else {
+                        reach = fmaxf(reach, scan_word(*reinterpret_cast<const uint16_t *>(blk + scale_offset<TYPE>())));
+                    }
+                }
+            }
+            reach = fmaxf(reach, __shfl_xor(reach, 32));
+            int exponent = static_cast<int>(__float_as_uint(reach) >> 23);   // biased
+            exponent = min(max(exponent, 9), 254);
+            if (half == 0) {
+                lds.row_power[c.item & 1][32 * dw + l32] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^S
+            }
+            return __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-S
+        };
 
         // Packed blocks of FSC_RAW_DEPTH super-blocks are in flight in registers: a lone request per super-block would
         // leave the wave waiting for memory once per super-block.
@@ -192,24 +321,24 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             WideRegs<WIDE_REGS> wide;
         };
         RawSet ring[FSC_RAW_DEPTH];
-        auto request = [&](int kb, RawSet & set) {
+        auto request = [&](const Cursor & c, RawSet & set) {
             if constexpr (K45) {
-                const uint8_t * base = wave_weights + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+                const uint8_t * base = c.rows + static_cast<int64_t>(c.kb) * F::BLOCK_BYTES;
 #pragma unroll
                 for (int i = 0; i < RAW_REGS; ++i) {
                     // ids past the wave's blocks repeat the last unit, so no lane branches around a load
                     const int id = min(lane + 64 * i, 32 * RAW_UNITS - 1);
                     const int row = id / RAW_UNITS;
                     const int unit = id - row * RAW_UNITS;
-                    const uint32_t offset = __umul24(min(row, rows_valid - 1), static_cast<uint32_t>(a.row_bytes)) + unit * 16;
+                    const uint32_t offset = __umul24(min(row, c.rows_valid - 1), static_cast<uint32_t>(a.row_bytes)) + unit * 16;
                     set.units[i] = *reinterpret_cast<const u32x4_t *>(base + offset);
                 }
             } else if constexpr (WIDE) {
-                wide_fetch<TYPE, 32, 64, WIDE_REGS>(set.wide, wave_weights, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
+                wide_fetch<TYPE, 32, 64, WIDE_REGS>(set.wide, c.rows, static_cast<int>(a.row_bytes), c.rows_valid, c.kb, lane);
             }
         };
-        // `kb`: the super-block the registers were requested for; `slot_parity`: where it goes
-        auto park = [&](int kb, int slot_parity, const RawSet & set) {
+        // `c`: the super-block the registers were requested for; `slot_parity`: where it goes
+        auto park = [&](const Cursor & c, int slot_parity, const RawSet & set) {
             uint8_t * const slot = lds.raw[dw][slot_parity];
             if constexpr (K45) {
 #pragma unroll
@@ -218,23 +347,23 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
                     *reinterpret_cast<u32x4_t *>(slot + id * 16) = set.units[i];   // (slots lie back to back: row * BLOCK_BYTES + unit * 16)
                 }
             } else if constexpr (WIDE) {
-                wide_park<TYPE, 32, 64, WIDE_REGS>(slot, set.wide, wave_weights, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
+                wide_park<TYPE, 32, 64, WIDE_REGS>(slot, set.wide, c.rows, static_cast<int>(a.row_bytes), c.rows_valid, c.kb, lane);
             } else {
-                stage_blocks<TYPE>(slot, weights, a.row_bytes, n0 + 32 * dw, a.out_features, kb, 32, lane, 64);
+                stage_blocks<TYPE>(slot, c.weights, a.row_bytes, c.n0 + 32 * dw, a.out_features, c.kb, 32, lane, 64);
             }
         };
         // A lane keeps weight row `l32` of the wave's 32 and takes k-half `half` of every 32-value block.
         const uint32_t out_lane = static_cast<uint32_t>(dw * (FSC_STEPS * 1024) + half * 1024 + l32 * 16);
-        auto block_of = [&](int kb) { return lds.raw[dw][kb & 1] + l32 * SLOT_PITCH + SLOT_FRONT; };
+        auto block_of = [&](int parity) { return lds.raw[dw][parity] + l32 * SLOT_PITCH + SLOT_FRONT; };
         // Q4_K/Q5_K: what a stage's unpack reads from the parked block, fetched a phase before it is used (a lone
         // wave has nothing else to cover an LDS round trip with): the 16-byte header (d, dmin, 12 bytes of 6-bit
         // scales and minima), this k-half's fifth-bit bytes, and its 16 bytes of each of the stage's two nibble chunks.
         struct StageInputs {
             u32x4_t header, planes, nibbles[2];
         };
-        auto fetch_inputs = [&](int stage_of_block, int kb) {
+        auto fetch_inputs = [&](int stage_of_block, int parity) {
             constexpr int QS = TYPE == Q4_K ? 16 : 48;
-            const uint8_t * blk = block_of(kb);
+            const uint8_t * blk = block_of(parity);
             StageInputs in;
             in.header = *reinterpret_cast<const u32x4_t *>(blk);
             in.planes = u32x4_t{0, 0, 0, 0};
@@ -245,6 +374,7 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             in.nibbles[1] = *reinterpret_cast<const u32x4_t *>(blk + QS + (2 * stage_of_block + 1) * 32 + 16 * half);
             return in;
         };
+        float shrink = 1.0f;   // 2^-S of the lane's weight row in the item being unpacked
         // the eight block minima of a Q4_K/Q5_K super-block as the operand of its extra reduction step
         auto minima_from_header = [&](int parity, const u32x4_t header) {
             int sc, mn[8];
@@ -311,11 +441,11 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             chunk(std::integral_constant<int, 0>{});
             chunk(std::integral_constant<int, 1>{});
         };
-        // the other formats: stage S of super-block kb straight from the parked block
-        auto unpack = [&](auto stage_tag, int kb, int target) {
+        // the other formats: stage S of the super-block parked in slot `parity`
+        auto unpack = [&](auto stage_tag, int parity, int target) {
             constexpr int S = decltype(stage_tag)::value;
             if constexpr (!K45) {
-                const uint8_t * blk = block_of(kb);
+                const uint8_t * blk = block_of(parity);
                 uint8_t * const out = &lds.wq[target][0] + out_lane;
                 const auto * const grid = &lds.codebook;
                 const _Float16 h = static_cast<_Float16>(half_weight_scale<TYPE>(blk) * shrink);
@@ -340,57 +470,37 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             }
         };
 
-        // The multiplying waves request their activation fragments a few reduction steps ahead, which covers a trip to
-        // L2 but not one to HBM; this wave therefore touches, FSC_TOUCH_AHEAD stages ahead, one word of every 128-byte
-        // line that two of the task's 32-row tiles will need (tiles first + 2 dw and + 2 dw + 1; wave 0 also a ninth
-        // one that an unaligned task reaches into), so that the lines wait in L2.  The words are summed into a value
-        // that is never used for anything else.
-        const int stages = 2 * super_blocks;
-        const int first_tile = row_start >> 5;
-        const int last_tile = (min(row_end, a.rows_padded) - 1) >> 5;
-        const int64_t tile_stride = static_cast<int64_t>(a.in_features / 32) * 2048;
-        const uint8_t * const touch_base[3] = {
-            reinterpret_cast<const uint8_t *>(a.qx) + min(first_tile + 2 * dw, last_tile) * tile_stride,
-            reinterpret_cast<const uint8_t *>(a.qx) + min(first_tile + 2 * dw + 1, last_tile) * tile_stride,
-            reinterpret_cast<const uint8_t *>(a.qx) + min(first_tile + 8, last_tile) * tile_stride};
-        uint32_t touched[FSC_TOUCH_AHEAD][3];
-        uint32_t touch_sink = 0;
-        auto touch = [&](int stage_index, uint32_t (&words)[3]) {
-            const int64_t offset = static_cast<int64_t>(min(stage_index, stages - 1)) * (FSC_STEPS * 1024) + lane * 128;
-            words[0] = *reinterpret_cast<const uint32_t *>(touch_base[0] + offset);
-            words[1] = *reinterpret_cast<const uint32_t *>(touch_base[1] + offset);
-            words[2] = dw == 0 ? *reinterpret_cast<const uint32_t *>(touch_base[2] + offset) : 0u;
-        };
-        auto touch_advance = [&](int stage_index) {
-            touch_sink += touched[0][0] + touched[0][1] + touched[0][2];
-#pragma unroll
-            for (int ahead = 0; ahead + 1 < FSC_TOUCH_AHEAD; ++ahead) {
-#pragma unroll
-                for (int i = 0; i < 3; ++i) {
-                    touched[ahead][i] = touched[ahead + 1][i];
-                }
-            }
-            touch(stage_index + FSC_TOUCH_AHEAD, touched[FSC_TOUCH_AHEAD - 1]);
-        };
-#pragma unroll
-        for (int ahead = 0; ahead < FSC_TOUCH_AHEAD; ++ahead) {
-            touch(1 + ahead, touched[ahead]);
-        }
-        const int last = super_blocks - 1;
+
+        // c_request walks FSC_RAW_DEPTH super-blocks ahead of c_park, which is one ahead of the super-block the
+        // multipliers work on; c_scan is the item whose scale words are in flight.
+        Cursor c_request, c_park, c_scan;
+        open_item(c_request, 0);
+        open_item(c_park, 0);
+        open_item(c_scan, 0);
 #pragma unroll
         for (int ahead = 0; ahead < FSC_RAW_DEPTH; ++ahead) {
-            request(min(ahead, last), ring[ahead]);
+            request(c_request, ring[ahead]);
+            step(c_request);
         }
+        uint32_t scan_words[SCAN_REGS];
+        scan_request(c_scan, scan_words);
+        shrink = scan_finish(c_scan, scan_words);
+        if (n_items > 1) {
+            open_item(c_scan, 1);
+        }
+        scan_request(c_scan, scan_words);
         // the oldest set goes to LDS, the others move up, the newest is requested
-        auto advance = [&](int parked_kb, int slot_parity, int requested_kb) {
-            park(parked_kb, slot_parity, ring[0]);
+        auto advance = [&](int slot_parity) {
+            park(c_park, slot_parity, ring[0]);
+            step(c_park);
 #pragma unroll
             for (int ahead = 0; ahead + 1 < FSC_RAW_DEPTH; ++ahead) {
                 ring[ahead] = ring[ahead + 1];
             }
-            request(requested_kb, ring[FSC_RAW_DEPTH - 1]);
+            request(c_request, ring[FSC_RAW_DEPTH - 1]);
+            step(c_request);
         };
-        advance(0, 0, min(FSC_RAW_DEPTH, last));
+        advance(0);
         StageInputs inputs = {};
         if constexpr (K45) {
             inputs = fetch_inputs(0, 0);
@@ -403,126 +513,122 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         FSC_LAP(0);
         __syncthreads();
         FSC_LAP(1);
+        int kb = 0;   // of super-block q within its item
 #pragma unroll 1
-        for (int kb = 0; kb < super_blocks; ++kb) {
+        for (int q = 0; q < total; ++q) {
+            const int parity = q & 1;
             // (past the last super-block the wave works on a repeat of it: nobody reads what that writes)
-            // while the multipliers work on stage 0 of kb: stage 1 of kb, then the next super-block's blocks
-#ifndef FSC_NO_UNPACK
+            // while the multipliers work on stage 0 of q: stage 1 of q, then the next super-block's blocks
             if constexpr (K45) {
                 finish_stage(std::integral_constant<int, 1>{}, inputs, 1);
             } else {
-                unpack(std::integral_constant<int, 1>{}, kb, 1);
+                unpack(std::integral_constant<int, 1>{}, parity, 1);
             }
-#endif
-            FSC_LAP(4);
-            advance(min(kb + 1, last), (kb + 1) & 1, min(kb + 1 + FSC_RAW_DEPTH, last));
             FSC_LAP(2);
-            touch_advance(2 * kb + 1);
+            advance(parity ^ 1);
             FSC_LAP(3);
             if constexpr (K45) {
-                inputs = fetch_inputs(0, kb + 1);
+                inputs = fetch_inputs(0, parity ^ 1);
             }
             __syncthreads();
-            FSC_LAP(5);
-            // while they work on stage 1: stage 0 of kb + 1
-#ifndef FSC_NO_UNPACK
-            if constexpr (K45) {
-                minima_from_header((kb + 1) & 1, inputs.header);
-                finish_stage(std::integral_constant<int, 0>{}, inputs, 0);
-                inputs = fetch_inputs(1, kb + 1);
+            FSC_LAP(4);
+            // while they work on stage 1: stage 0 of q + 1, which may open the next item
+            if (kb + 1 == super_blocks) {
+                kb = 0;
+                if (q + 1 < total) {
+                    shrink = scan_finish(c_scan, scan_words);
+                    if (c_scan.item + 1 < n_items) {
+                        open_item(c_scan, c_scan.item + 1);
+                    }
+                    scan_request(c_scan, scan_words);
+                }
             } else {
-                unpack(std::integral_constant<int, 0>{}, kb + 1, 0);
+                ++kb;
             }
-#endif
-            FSC_LAP(6);
-            touch_advance(2 * kb + 2);
-            FSC_LAP(3);
-            __syncthreads();
             FSC_LAP(5);
+            if constexpr (K45) {
+                minima_from_header(parity ^ 1, inputs.header);
+                finish_stage(std::integral_constant<int, 0>{}, inputs, 0);
+                inputs = fetch_inputs(1, parity ^ 1);
+            } else {
+                unpack(std::integral_constant<int, 0>{}, parity ^ 1, 0);
+            }
+            FSC_LAP(6);
+            __syncthreads();
+            FSC_LAP(4);
         }
-#pragma unroll
-        for (int ahead = 0; ahead < FSC_TOUCH_AHEAD; ++ahead) {
-            touch_sink += touched[ahead][0] + touched[ahead][1] + touched[ahead][2];
-        }
-        if (touch_sink == 0x5ca1ab1eu && a.rows < 0) {   // (never true: keeps the touches alive)
-            lds.row_power[lane] = 1.0f;
-        }
-        __syncthreads();
-#ifdef FSC_TIMING
-        if (profiled >= 0 && lane == 0) { for (int i = 0; i < 8; ++i) fsc_times[profiled][1][i + 1] = lap[i]; }
-#endif
+        FSC_LAP_DUMP(1);
         return;
     }
 
     // ---------------- multiplying wave ----------------
-#ifdef FSC_MULT_PRIO
-    __builtin_amdgcn_s_setprio(FSC_MULT_PRIO);
-#endif
-    const int wave_row = row_start + wave * 64;
-    const bool wave_active = wave_row < row_end;
-    if (!wave_active) {
-        __syncthreads();
-#pragma unroll 1
-        for (int kb = 0; kb < super_blocks; ++kb) {
-            __syncthreads();
-            __syncthreads();
-        }
-        __syncthreads();
-        return;
-    }
     // Every global address is a uniform 64-bit base, advanced with scalar arithmetic, plus a 32-bit lane offset.
     const int blocks_per_row = a.in_features / 32;
-    const int total_steps = a.in_features / 16;
-    const int first_tile = row_start >> 5;
-    const uint8_t * const qx_task = reinterpret_cast<const uint8_t *>(a.qx) + static_cast<int64_t>(first_tile) * blocks_per_row * 2048;
-    const uint8_t * const sums_task = reinterpret_cast<const uint8_t *>(a.block_sums) + static_cast<int64_t>(first_tile) * super_blocks * 512;
-    uint32_t x_lane_offset[2], sums_lane_offset[2];
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        int lane_row = wave_row + 32 * rt + l32;
-        lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
-        x_lane_offset[rt] = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
-                            static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
-        sums_lane_offset[rt] = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
-                               static_cast<uint32_t>((lane_row & 31) * 16);
-    }
-
-    // reduction step G (16 values) of the task's rows: one 1 KiB slab per 32-row tile
-    auto load_x = [&](int step, half8_t (&out)[2]) {
-#ifdef FSC_X_HOT
-        const int clamped = step & 7;
-#else
-        const int clamped = step < total_steps ? step : total_steps - 1;
-#endif
-        const uint8_t * base = qx_task + static_cast<int64_t>(clamped) * 1024;
-        out[0] = *reinterpret_cast<const half8_t *>(base + x_lane_offset[0]);
-        out[1] = *reinterpret_cast<const half8_t *>(base + x_lane_offset[1]);
+    // Where this wave's activation rows of an item are: a wave without rows in the item multiplies the workspace's
+    // last rows instead (no branch around the matrix instructions; nothing of it is stored).
+    struct Rows {
+        const uint8_t * x;      // fragment slabs of the item's first 32-row tile
+        const uint8_t * sums;   // block sums of the same tile
+        uint32_t x_lane[2], sums_lane[2], power_lane[2];
     };
-    auto load_sums = [&](int kb, uint4 (&out)[2]) {
-        const int clamped = kb < super_blocks ? kb : super_blocks - 1;
-        const uint8_t * base = sums_task + static_cast<int64_t>(clamped) * 512;
-        out[0] = *reinterpret_cast<const uint4 *>(base + sums_lane_offset[0]);
-        out[1] = *reinterpret_cast<const uint4 *>(base + sums_lane_offset[1]);
+    auto rows_of = [&](int item) {
+        Rows r;
+        const int row_start = item_field(item, 1);
+        const int first_tile = row_start >> 5;
+        r.x = reinterpret_cast<const uint8_t *>(a.qx) + static_cast<int64_t>(first_tile) * blocks_per_row * 2048;
+        r.sums = reinterpret_cast<const uint8_t *>(a.block_sums) + static_cast<int64_t>(first_tile) * super_blocks * 512;
+#pragma unroll
+        for (int rt = 0; rt < 2; ++rt) {
+            int lane_row = row_start + wave * 64 + 32 * rt + l32;
+            lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
+            r.x_lane[rt] = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
+                           static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
+            r.sums_lane[rt] = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
+                              static_cast<uint32_t>((lane_row & 31) * 16);
+            r.power_lane[rt] = static_cast<uint32_t>(lane_row) * 4u;
+        }
+        return r;
+    };
+    // reduction step `step` (16 values) of the rows: one 1 KiB slab per 32-row tile
+    auto load_x = [&](const Rows & r, int step, half8_t (&out)[2]) {
+        const uint8_t * base = r.x + static_cast<int64_t>(step) * 1024;
+        out[0] = *reinterpret_cast<const half8_t *>(base + r.x_lane[0]);
+        out[1] = *reinterpret_cast<const half8_t *>(base + r.x_lane[1]);
+    };
+    // 2^(e - E) of the lane's two rows in super-block kb, as fp16 pairs: what brings the super-block's fragments, which
+    // the quantizer normalised by themselves, to the row's common exponent (a power of two: exact; a super-block
+    // more than 2^24 below the row's largest one vanishes)
+    auto load_ratio = [&](const Rows & r, int kb, float (&out)[2]) {
+        const uint8_t * base = reinterpret_cast<const uint8_t *>(a.power + static_cast<int64_t>(kb) * a.rows_padded);
+        out[0] = *reinterpret_cast<const float *>(base + r.power_lane[0]);
+        out[1] = *reinterpret_cast<const float *>(base + r.power_lane[1]);
+    };
+    auto rescale = [&](half8_t fragment, half2_t ratio) {
+        const uint4 words = __builtin_bit_cast(uint4, fragment);
+        const uint4 scaled = make_uint4(half2_mul(words.x, ratio), half2_mul(words.y, ratio), half2_mul(words.z, ratio),
+                                        half2_mul(words.w, ratio));
+        return __builtin_bit_cast(half8_t, scaled);
+    };
+    auto load_sums = [&](const Rows & r, int kb, uint4 (&out)[2]) {
+        const uint8_t * base = r.sums + static_cast<int64_t>(kb) * 512;
+        out[0] = *reinterpret_cast<const uint4 *>(base + r.sums_lane[0]);
+        out[1] = *reinterpret_cast<const uint4 *>(base + r.sums_lane[1]);
     };
 
-    // activation fragments are requested FSC_X_AHEAD reduction steps before their matrix instructions
-    half8_t x[FSC_X_AHEAD][2];
+    // activation fragments are requested a whole stage (FSC_STEPS reduction steps) before their matrix instructions
+    Rows rows_next = rows_of(0);   // of the stage being requested
+    half8_t x[FSC_STEPS][2];
 #pragma unroll
-    for (int i = 0; i < FSC_X_AHEAD; ++i) {
-        load_x(i, x[i]);
-    }
-    uint4 sums[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
-    if constexpr (K45) {
-        load_sums(0, sums);
+    for (int i = 0; i < FSC_STEPS; ++i) {
+        load_x(rows_next, i, x[i]);
     }
 
     v16f acc[2][FWD_NT];
+    const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
     for (int rt = 0; rt < 2; ++rt)
 #pragma unroll
-        for (int nt = 0; nt < FWD_NT; ++nt)
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[rt][nt][v] = 0.0f;
+        for (int nt = 0; nt < FWD_NT; ++nt) acc[rt][nt] = zero;
 
     // weight fragments are read FSC_W_AHEAD reduction steps before their matrix instructions
     constexpr int RING = FSC_W_AHEAD + 1;
@@ -533,26 +639,28 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             out[nt] = *reinterpret_cast<const half8_t *>(&lds.wq[buffer][((nt * FSC_STEPS + step) * 64 + lane) * 16]);
         }
     };
-    static_assert(FSC_STEPS % FSC_X_AHEAD == 0, "a stage starts at slot 0 of the activation ring");
-    // one stage: eight reduction steps from operand tile `buffer` (its first FSC_W_AHEAD steps have been read)
-    auto stage = [&](int buffer, int first_step) {
+    // one stage: eight reduction steps from operand tile `buffer` (its first FSC_W_AHEAD steps have been read); every
+    // step's activation registers are refilled with the same step of the following stage (`next_step` of `rows_next`)
+    auto stage = [&](int buffer, int next_step, const half2_t (&ratio)[2]) {
 #pragma unroll
         for (int s = 0; s < FSC_STEPS; ++s) {
-#ifndef FSC_NO_AREAD
             if (s + FSC_W_AHEAD < FSC_STEPS) {
                 read_step(buffer, s + FSC_W_AHEAD, w[(s + FSC_W_AHEAD) % RING]);
             }
-#endif
 #pragma unroll
             for (int rt = 0; rt < 2; ++rt) {
+                const half8_t fragment = rescale(x[s][rt], ratio[rt]);
 #pragma unroll
                 for (int nt = 0; nt < FWD_NT; ++nt) {
-                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(x[s % FSC_X_AHEAD][rt], w[s % RING][nt], acc[rt][nt], 0, 0, 0);
+                    // (weights as the A operand: the lane ends up with one activation row and runs of four neighbouring
+                    // columns, which the epilogue stages with 8-byte LDS writes)
+                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[s % RING][nt], fragment, acc[rt][nt], 0, 0, 0);
                 }
             }
-#ifndef FSC_NO_XLOAD
-            load_x(first_step + s + FSC_X_AHEAD, x[s % FSC_X_AHEAD]);
-#endif
+            load_x(rows_next, next_step + s, x[s]);
+            // (the requests stay where they are written: moved to the end of the stage, as the scheduler would have
+            // them, they leave the next stage waiting for memory)
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     auto read_first_steps = [&](int buffer) {
@@ -565,83 +673,102 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
     __syncthreads();
     FSC_LAP(1);
     read_first_steps(0);
+    int item = 0, kb = 0;
 #pragma unroll 1
-    for (int kb = 0; kb < super_blocks; ++kb) {
-        uint4 sums_next[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+    for (int q = 0; q < total; ++q) {
+        // (rows_next: still the rows of this super-block's item, whose stage 0 was requested with them)
+        uint4 sums[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
         if constexpr (K45) {
-            load_sums(kb + 1, sums_next);
+            load_sums(rows_next, kb, sums);
         }
-        stage(0, kb * 16);
+        float ratio_f32[2];
+        load_ratio(rows_next, kb, ratio_f32);
+        const half2_t ratio[2] = {half2_t{static_cast<_Float16>(ratio_f32[0]), static_cast<_Float16>(ratio_f32[0])},
+                                  half2_t{static_cast<_Float16>(ratio_f32[1]), static_cast<_Float16>(ratio_f32[1])}};
+        // stage 0; requests stage 1 of the same super-block
+        stage(0, kb * 16 + 8, ratio);
         FSC_LAP(2);
         __syncthreads();
         FSC_LAP(3);
         read_first_steps(1);
-        stage(1, kb * 16 + 8);
+        // stage 1; requests stage 0 of the following super-block, which may belong to the next item
+        const bool last_of_item = kb + 1 == super_blocks;
+        const int item_next = last_of_item ? min(item + 1, n_items - 1) : item;
+        const int kb_next = last_of_item ? 0 : kb + 1;
+        rows_next = rows_of(item_next);
+        stage(1, kb_next * 16, ratio);
         if constexpr (K45) {
-            // the super-block's extra reduction step: block sums x block minima (slots 8..15 of the instruction are empty)
+            // the super-block's extra reduction step: block minima x block sums (slots 8..15 of the instruction are empty)
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) {
-                uint4 minima = *reinterpret_cast<const uint4 *>(&lds.mins[kb & 1][nt * 512 + l32 * 16]);
+                uint4 minima = *reinterpret_cast<const uint4 *>(&lds.mins[q & 1][nt * 512 + l32 * 16]);
                 if (half != 0) {
                     minima = make_uint4(0, 0, 0, 0);
                 }
 #pragma unroll
                 for (int rt = 0; rt < 2; ++rt) {
                     const uint4 block_sums = half != 0 ? make_uint4(0, 0, 0, 0) : sums[rt];
-                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, block_sums),
-                                                                         __builtin_bit_cast(half8_t, minima), acc[rt][nt], 0, 0, 0);
+                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, minima),
+                                                                         rescale(__builtin_bit_cast(half8_t, block_sums), ratio[rt]),
+                                                                         acc[rt][nt], 0, 0, 0);
                 }
             }
-            sums[0] = sums_next[0];
-            sums[1] = sums_next[1];
         }
         FSC_LAP(4);
         __syncthreads();
         FSC_LAP(3);
-        read_first_steps(0);   // of the next super-block (a stale tile after the last one: never used)
-    }
-    __syncthreads();
-    FSC_LAP(6);
-
-    // The operand tiles are free now: each wave scales its results by 2^(E[r] + S[n]), transposes them 32 rows at a
-    // time through its share of that memory (rows padded to 136) and writes whole 256-byte rows.
-    constexpr int STAGE_PITCH = 136;
-    static_assert(sizeof(lds.wq) >= 4 * 32 * STAGE_PITCH * sizeof(uint16_t), "the staging area fits");
-    uint16_t * const stage_base = reinterpret_cast<uint16_t *>(&lds.wq[0][0]);
-    typedef float float4_unaligned __attribute__((ext_vector_type(4), aligned(4)));
-    float column_power[FWD_NT];
+        if (last_of_item) {
+            // The item is complete: scale by 2^(E[r] + S[n]) and store, 32 rows x 64 columns at a time through this
+            // wave's staging area, while the unpacking waves work on the next item.
+            const int row_start = item_field(item, 1);
+            const int row_end = item_field(item, 2);
+            const int tile = item_field(item, 3);
+            const bool second = tile >= a.n_tiles;
+            const int n0 = (second ? tile - a.n_tiles : tile) * FWD_TN;
+            uint16_t * const y = second ? a.y_second : a.y;
+            const int wave_row = row_start + wave * 64;
+            // recomputing the lane's share here is cheaper than keeping it alive through the loop
+            int lane_here = lane;
+            asm volatile("" : "+v"(lane_here));
+            const int l32_here = lane_here & 31, half_here = lane_here >> 5;
 #pragma unroll
-    for (int nt = 0; nt < FWD_NT; ++nt) {
-        column_power[nt] = lds.row_power[nt * 32 + l32];
-    }
+            for (int rt = 0; rt < 2; ++rt) {
+                const int r0 = wave_row + 32 * rt;
+                if (r0 < row_end) {
+                    const float row_power = a.row_power[min(r0 + l32_here, a.rows_padded - 1)];
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int r0 = wave_row + 32 * rt;
-        if (r0 < row_end) {
-            // the lane's rows r0 + 8 j + 4 half + 0..3 (rows past the workspace read on into the plane's successor:
-            // their results are never stored)
-            const float * powers = a.power + r0 + 4 * half;
+                    for (int pair = 0; pair < 2; ++pair) {
 #pragma unroll
-            for (int j = 0; j < 4; ++j) {
-                const float4_unaligned run = *reinterpret_cast<const float4_unaligned *>(powers + 8 * j);
-                const float row_power[4] = {run.x, run.y, run.z, run.w};
+                        for (int t = 0; t < 2; ++t) {
+                            const int nt = 2 * pair + t;
 #pragma unroll
-                for (int nt = 0; nt < FWD_NT; ++nt) {
-#pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        acc[rt][nt][4 * j + i] *= row_power[i] * column_power[nt];
+                            for (int j = 0; j < 4; ++j) {
+                                const float4 column_power =
+                                    *reinterpret_cast<const float4 *>(&lds.row_power[item & 1][nt * 32 + 8 * j + 4 * half_here]);
+                                acc[rt][nt][4 * j + 0] *= row_power * column_power.x;
+                                acc[rt][nt][4 * j + 1] *= row_power * column_power.y;
+                                acc[rt][nt][4 * j + 2] *= row_power * column_power.z;
+                                acc[rt][nt][4 * j + 3] *= row_power * column_power.w;
+                            }
+                        }
+                        const v16f (&tiles)[2] = *reinterpret_cast<const v16f (*)[2]>(&acc[rt][2 * pair]);
+                        store_rows_32x64(lds.staging[wave], tiles,
+                                         y + static_cast<int64_t>(r0) * a.out_features + n0 + 64 * pair, a.out_features,
+                                         row_end - r0, a.out_features - n0 - 64 * pair, lane_here);
                     }
                 }
+#pragma unroll
+                for (int nt = 0; nt < FWD_NT; ++nt) acc[rt][nt] = zero;
             }
-            const int64_t origin = static_cast<int64_t>(r0) * a.out_features + n0;
-            store_rows_32x128<STAGE_PITCH, false, false>(stage_base + wave * (32 * STAGE_PITCH), acc[rt], y + origin, a.out_features,
-                                                         row_end - r0, a.out_features - n0, lane, nullptr);
+            ++item;
+            kb = 0;
+            FSC_LAP(5);
+        } else {
+            ++kb;
         }
+        read_first_steps(0);   // of the next super-block (a stale tile after the last one: never used)
     }
-#ifdef FSC_TIMING
-    FSC_LAP(7);
-    if (profiled >= 0 && lane == 0) { fsc_times[profiled][0][94] = wall_clock64(); for (int i = 0; i < 8; ++i) fsc_times[profiled][0][i + 1] = lap[i]; }
-#endif
+    FSC_LAP_DUMP(0);
 }
 
 #ifdef FSC_TIMING
@@ -657,14 +784,23 @@ static hipError_t launch_forward_scaled_typed(const ForwardArgs & args, hipStrea
     if (total <= 0 || total > 0x7fffffffLL || args.swiglu != 0 || args.in_features > (1 << 22)) {
         return hipErrorInvalidValue;
     }
+    // one workgroup per CU; more when a workgroup's table would not hold its share (a multiple of the XCD count
+    // either way, so that a workgroup's items stay on its XCD)
+    int64_t grid = FSC_GRID;
+    if (total > grid * FSC_MAX_ITEMS) {
+        grid = ((total + FSC_MAX_ITEMS - 1) / FSC_MAX_ITEMS + XCDS - 1) / XCDS * XCDS;
+    }
+    if (total < grid) {
+        grid = total;
+    }
     const ProfileScope scope(2, stream);
     if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
         if (args.wide != 0) {
-            mmq_forward_scaled_kernel<TYPE, true><<<static_cast<unsigned>(total), FSC_THREADS, 0, stream>>>(args);
+            mmq_forward_scaled_kernel<TYPE, true><<<static_cast<unsigned>(grid), FSC_THREADS, 0, stream>>>(args, static_cast<int>(total));
             return hipGetLastError();
         }
     }
-    mmq_forward_scaled_kernel<TYPE, false><<<static_cast<unsigned>(total), FSC_THREADS, 0, stream>>>(args);
+    mmq_forward_scaled_kernel<TYPE, false><<<static_cast<unsigned>(grid), FSC_THREADS, 0, stream>>>(args, static_cast<int>(total));
     return hipGetLastError();
 }
 

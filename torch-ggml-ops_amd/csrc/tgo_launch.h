@@ -104,8 +104,9 @@ struct Q8Workspace {
                     // half and scaled tiles: [rows_padded/32][K/32][2 k-halves][2 eighths x 32 rows][8 fp16]
     float * d;      // tiles: [K/32][rows_padded]                                         rows: [rows][K/32]
     float * sum;    // same as d
-    float * power;  // scaled tiles: 2^E per row, [rows_padded]
-    uint16_t * block_sums;   // scaled tiles: fp16(sum * 2^-E) per block, [rows_padded/32][K/256][32 rows][8 blocks]
+    float * power;  // scaled tiles: 2^(e - E) per row and super-block, [K/256][rows_padded] (2^e until the second pass)
+    uint16_t * block_sums;   // scaled tiles: fp16(sum * 2^-e) per block, [rows_padded/32][K/256][32 rows][8 blocks]
+    float * row_power;       // scaled tiles: 2^E per row, [rows_padded]
     uint32_t * tag;          // WORKSPACE_TAG_MAGIC | layout, written by the quantizer
     int64_t rows_padded;
     int layout;
@@ -125,7 +126,8 @@ static inline int64_t q8_workspace_bytes(int64_t rows, int64_t in_features) {
     // the 1 KiB tail lets kernels fetch the scales of a whole 32-row tile with 16-byte loads even when the
     // tile starts at the last row; its first word is the layout tag
     return 2 * padded * in_features + 2 * padded * (in_features / 32) * static_cast<int64_t>(sizeof(float)) +
-           padded * (in_features / 256) * (static_cast<int64_t>(sizeof(float)) + 16) + 1024;
+           padded * (in_features / 256) * (static_cast<int64_t>(sizeof(float)) + 16) +
+           padded * static_cast<int64_t>(sizeof(float)) + 1024;
 }
 
 // `operand_kind`: OPERAND_INT8, OPERAND_HALF or OPERAND_SCALED (forward_operand_kind); ignored for by_rows.
@@ -140,7 +142,8 @@ static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t i
     view.sum = view.d + view.rows_padded * (in_features / 32);
     view.power = view.sum + view.rows_padded * (in_features / 32);
     view.block_sums = reinterpret_cast<uint16_t *>(view.power + view.rows_padded * (in_features / 256));
-    view.tag = reinterpret_cast<uint32_t *>(reinterpret_cast<uint8_t *>(view.block_sums) + view.rows_padded * (in_features / 256) * 16);
+    view.row_power = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(view.block_sums) + view.rows_padded * (in_features / 256) * 16);
+    view.tag = reinterpret_cast<uint32_t *>(view.row_power + view.rows_padded);
     return view;
 }
 

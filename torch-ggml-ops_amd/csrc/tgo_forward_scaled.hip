@@ -17,13 +17,13 @@
 // first and the last reduction step.  The int8 kernels spend two or three vector operations per result on every 32
 // values, which bounds them at a quarter of the matrix pipe's rate.
 //
-// Work split: role-split workgroup of eight waves, one per CU.  Waves 0-3 multiply: wave w owns activation rows
-// [64w, 64w + 64) of the task and all 128 weight rows of the column tile (2 x 4 tiles of 32 x 32, 128 accumulator
-// registers; the activations are the A operand, so a lane holds one weight row per tile and 16 activation rows).
-// Waves 4-7 unpack: wave 4 + t owns weight rows [32t, 32t + 32) from the global load of their packed blocks to
-// their fp16 operand tile (packed blocks FSC_RAW_DEPTH super-blocks ahead in registers, parked in the wave's own LDS
-// slot; LDS executes a wave's accesses in order, so these steps need no workgroup barrier).  Each SIMD then holds one
-// wave that feeds the matrix pipe and one that keeps the vector pipe busy.  A super-block is two stages of 128
+// Work split: role-split workgroup of twelve waves, one per CU.  Waves 0-7 multiply: wave w owns activation rows
+// [32w, 32w + 32) of the task and all 128 weight rows of the column tile (1 x 4 tiles of 32 x 32, 64 accumulator
+// registers; the weights are the A operand, so a lane holds one activation row and 16 weight rows per tile).
+// Waves 8-11 unpack: wave 8 + t owns weight rows [32t, 32t + 32) from the global load of their packed blocks to
+// their fp16 operand tile (packed blocks RAW_DEPTH super-blocks ahead in registers, parked in the wave's own LDS
+// slot; LDS executes a wave's accesses in order, so these steps need no workgroup barrier).  Each SIMD then holds two
+// waves that feed the matrix pipe and one that keeps the vector pipe busy.  A super-block is two stages of 128
 // values; the operand tile of a stage (32 KiB, fragment order) is double buffered and one barrier per stage hands
 // it over: while the multipliers work on stage g, the unpackers write stage g + 1.
 //
@@ -42,19 +42,17 @@ namespace tgo {
 
 typedef float v16f __attribute__((ext_vector_type(16)));
 
-constexpr int FSC_THREADS = 512;
+constexpr int FSC_MULTIPLIERS = 8;                         // multiplying waves, 32 activation rows each
+constexpr int FSC_THREADS = 64 * (FSC_MULTIPLIERS + 4);
 constexpr int FSC_STEPS = 8;                                // 16-value reduction steps per stage
 constexpr int FSC_TILE_BYTES = FWD_NT * FSC_STEPS * 1024;   // fp16 operand of a stage: [tile][step][64 lanes][16 bytes]
 constexpr int FSC_ROWS = 256;                               // activation rows per task
 static_assert(FSC_ROWS == forward_row_tile(12, OPERAND_SCALED), "task rows match the workgroup");
-#ifndef FSC_RAW_DEPTH
-#define FSC_RAW_DEPTH 3
-#endif
 #ifndef FSC_TOUCH_AHEAD
 #define FSC_TOUCH_AHEAD 4
 #endif
 #ifndef FSC_W_AHEAD
-#define FSC_W_AHEAD 2
+#define FSC_W_AHEAD 1
 #endif
 #ifndef FSC_X_AHEAD
 #define FSC_X_AHEAD 8
@@ -80,7 +78,7 @@ struct ScaledLds {
     alignas(16) uint8_t raw[4][2][32 * RAW_SLOT];              // per unpacking wave: packed blocks of two super-blocks
     alignas(16) uint8_t mins[2][K45 ? FWD_NT * 512 : 16];      // fp16(-dmin * m * 2^-S): [tile][32 rows][8 blocks], by parity
     alignas(16) float row_power[2][FWD_TN];                    // 2^S of the tile's weight rows, by the item's parity
-    alignas(16) uint16_t staging[4][32 * FSC_STAGE_PITCH];     // per multiplying wave: 32 rows x 64 columns of results
+    alignas(16) uint16_t staging[FSC_MULTIPLIERS][32 * FSC_STAGE_PITCH];   // per multiplying wave: 32 rows x 64 columns of results
     ScaledItem items[FSC_MAX_ITEMS];
     int item_count;
     std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;
@@ -173,7 +171,7 @@ TGO_DEVICE void store_rows_32x64(uint16_t * stage, const v16f (&tiles)[2], uint1
 }
 
 template <int TYPE, bool WIDE>
-__global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(const ForwardArgs a, const int total_slots) {
+__global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(const ForwardArgs a, const int total_slots) {
     using F = Format<TYPE>;
     using L = ScaledLds<TYPE>;
     constexpr bool K45 = L::K45;
@@ -215,7 +213,7 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         return;
     }
 #ifdef FSC_TIMING
-    const int profiled = (wave == 0 || wave == 4) && blockIdx.x % 32 == 5 ? blockIdx.x / 32 : -1;
+    const int profiled = (wave == 0 || wave == FSC_MULTIPLIERS) && blockIdx.x % 32 == 5 ? blockIdx.x / 32 : -1;
     unsigned long long lap[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     unsigned long long lap_last = __builtin_readcyclecounter();
     const unsigned long long wall_start = wall_clock64();
@@ -226,13 +224,15 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         return __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(&lds.items[item])[field]);
     };
 
-    if (wave >= 4) {
+    if (wave >= FSC_MULTIPLIERS) {
         // ---------------- unpacking wave ----------------
-        const int dw = wave - 4;
+        const int dw = wave - FSC_MULTIPLIERS;
         constexpr int RAW_UNITS = K45 ? F::BLOCK_BYTES / 16 : 1;
         constexpr int RAW_REGS = K45 ? (32 * RAW_UNITS + 63) / 64 : 1;
         using W = WideStage<TYPE>;
         constexpr int WIDE_REGS = WIDE ? W::template regs<32, 64>() : 1;
+        // super-blocks of packed blocks in flight in registers (Q6_K's 14 aligned units per block leave room for two)
+        constexpr int RAW_DEPTH = TYPE == Q6_K ? 2 : 3;
         constexpr int SLOT_PITCH = K45 ? F::BLOCK_BYTES : (WIDE ? W::PITCH : F::RAW_PITCH);
         constexpr int SLOT_FRONT = K45 ? 0 : (WIDE ? W::FRONT : F::RAW_SHIFT);
 
@@ -314,13 +314,13 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             return __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-S
         };
 
-        // Packed blocks of FSC_RAW_DEPTH super-blocks are in flight in registers: a lone request per super-block would
+        // Packed blocks of RAW_DEPTH super-blocks are in flight in registers: a lone request per super-block would
         // leave the wave waiting for memory once per super-block.
         struct RawSet {
             u32x4_t units[RAW_REGS];
             WideRegs<WIDE_REGS> wide;
         };
-        RawSet ring[FSC_RAW_DEPTH];
+        RawSet ring[RAW_DEPTH];
         auto request = [&](const Cursor & c, RawSet & set) {
             if constexpr (K45) {
                 const uint8_t * base = c.rows + static_cast<int64_t>(c.kb) * F::BLOCK_BYTES;
@@ -471,14 +471,14 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         };
 
 
-        // c_request walks FSC_RAW_DEPTH super-blocks ahead of c_park, which is one ahead of the super-block the
+        // c_request walks RAW_DEPTH super-blocks ahead of c_park, which is one ahead of the super-block the
         // multipliers work on; c_scan is the item whose scale words are in flight.
         Cursor c_request, c_park, c_scan;
         open_item(c_request, 0);
         open_item(c_park, 0);
         open_item(c_scan, 0);
 #pragma unroll
-        for (int ahead = 0; ahead < FSC_RAW_DEPTH; ++ahead) {
+        for (int ahead = 0; ahead < RAW_DEPTH; ++ahead) {
             request(c_request, ring[ahead]);
             step(c_request);
         }
@@ -494,10 +494,10 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             park(c_park, slot_parity, ring[0]);
             step(c_park);
 #pragma unroll
-            for (int ahead = 0; ahead + 1 < FSC_RAW_DEPTH; ++ahead) {
+            for (int ahead = 0; ahead + 1 < RAW_DEPTH; ++ahead) {
                 ring[ahead] = ring[ahead + 1];
             }
-            request(c_request, ring[FSC_RAW_DEPTH - 1]);
+            request(c_request, ring[RAW_DEPTH - 1]);
             step(c_request);
         };
         advance(0);
@@ -562,14 +562,16 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
     }
 
     // ---------------- multiplying wave ----------------
+    // Two of these share a SIMD: a lone wave issues a 32 x 32 x 16 matrix instruction only about every 42 cycles,
+    // two keep the pipe close to its 32.
     // Every global address is a uniform 64-bit base, advanced with scalar arithmetic, plus a 32-bit lane offset.
     const int blocks_per_row = a.in_features / 32;
-    // Where this wave's activation rows of an item are: a wave without rows in the item multiplies the workspace's
-    // last rows instead (no branch around the matrix instructions; nothing of it is stored).
+    // Where this wave's 32 activation rows of an item are: a wave without rows in the item reads the workspace's last
+    // rows instead and multiplies zeros (no branch around the matrix instructions; nothing of it is stored).
     struct Rows {
         const uint8_t * x;      // fragment slabs of the item's first 32-row tile
         const uint8_t * sums;   // block sums of the same tile
-        uint32_t x_lane[2], sums_lane[2], power_lane[2];
+        uint32_t x_lane, sums_lane, power_lane;
     };
     auto rows_of = [&](int item) {
         Rows r;
@@ -577,31 +579,25 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         const int first_tile = row_start >> 5;
         r.x = reinterpret_cast<const uint8_t *>(a.qx) + static_cast<int64_t>(first_tile) * blocks_per_row * 2048;
         r.sums = reinterpret_cast<const uint8_t *>(a.block_sums) + static_cast<int64_t>(first_tile) * super_blocks * 512;
-#pragma unroll
-        for (int rt = 0; rt < 2; ++rt) {
-            int lane_row = row_start + wave * 64 + 32 * rt + l32;
-            lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
-            r.x_lane[rt] = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
-                           static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
-            r.sums_lane[rt] = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
-                              static_cast<uint32_t>((lane_row & 31) * 16);
-            r.power_lane[rt] = static_cast<uint32_t>(lane_row) * 4u;
-        }
+        int lane_row = row_start + wave * 32 + l32;
+        lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
+        r.x_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
+                   static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
+        r.sums_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
+                      static_cast<uint32_t>((lane_row & 31) * 16);
+        r.power_lane = static_cast<uint32_t>(lane_row) * 4u;
         return r;
     };
     // reduction step `step` (16 values) of the rows: one 1 KiB slab per 32-row tile
-    auto load_x = [&](const Rows & r, int step, half8_t (&out)[2]) {
-        const uint8_t * base = r.x + static_cast<int64_t>(step) * 1024;
-        out[0] = *reinterpret_cast<const half8_t *>(base + r.x_lane[0]);
-        out[1] = *reinterpret_cast<const half8_t *>(base + r.x_lane[1]);
+    auto load_x = [&](const Rows & r, int step) {
+        return *reinterpret_cast<const half8_t *>(r.x + static_cast<int64_t>(step) * 1024 + r.x_lane);
     };
-    // 2^(e - E) of the lane's two rows in super-block kb, as fp16 pairs: what brings the super-block's fragments, which
-    // the quantizer normalised by themselves, to the row's common exponent (a power of two: exact; a super-block
-    // more than 2^24 below the row's largest one vanishes)
-    auto load_ratio = [&](const Rows & r, int kb, float (&out)[2]) {
+    // 2^(e - E) of the lane's row in super-block kb: what brings the super-block's fragments, which the quantizer
+    // normalised by themselves, to the row's common exponent (a power of two: exact; a super-block more than 2^24
+    // below the row's largest one vanishes)
+    auto load_ratio = [&](const Rows & r, int kb) {
         const uint8_t * base = reinterpret_cast<const uint8_t *>(a.power + static_cast<int64_t>(kb) * a.rows_padded);
-        out[0] = *reinterpret_cast<const float *>(base + r.power_lane[0]);
-        out[1] = *reinterpret_cast<const float *>(base + r.power_lane[1]);
+        return *reinterpret_cast<const float *>(base + r.power_lane);
     };
     auto rescale = [&](half8_t fragment, half2_t ratio) {
         const uint4 words = __builtin_bit_cast(uint4, fragment);
@@ -609,26 +605,22 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
                                         half2_mul(words.w, ratio));
         return __builtin_bit_cast(half8_t, scaled);
     };
-    auto load_sums = [&](const Rows & r, int kb, uint4 (&out)[2]) {
-        const uint8_t * base = r.sums + static_cast<int64_t>(kb) * 512;
-        out[0] = *reinterpret_cast<const uint4 *>(base + r.sums_lane[0]);
-        out[1] = *reinterpret_cast<const uint4 *>(base + r.sums_lane[1]);
+    auto load_sums = [&](const Rows & r, int kb) {
+        return *reinterpret_cast<const uint4 *>(r.sums + static_cast<int64_t>(kb) * 512 + r.sums_lane);
     };
 
     // activation fragments are requested a whole stage (FSC_STEPS reduction steps) before their matrix instructions
     Rows rows_next = rows_of(0);   // of the stage being requested
-    half8_t x[FSC_STEPS][2];
+    half8_t x[FSC_STEPS];
 #pragma unroll
     for (int i = 0; i < FSC_STEPS; ++i) {
-        load_x(rows_next, i, x[i]);
+        x[i] = load_x(rows_next, i);
     }
 
-    v16f acc[2][FWD_NT];
+    v16f acc[FWD_NT];
     const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt)
-#pragma unroll
-        for (int nt = 0; nt < FWD_NT; ++nt) acc[rt][nt] = zero;
+    for (int nt = 0; nt < FWD_NT; ++nt) acc[nt] = zero;
 
     // weight fragments are read FSC_W_AHEAD reduction steps before their matrix instructions
     constexpr int RING = FSC_W_AHEAD + 1;
@@ -640,24 +632,21 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         }
     };
     // one stage: eight reduction steps from operand tile `buffer` (its first FSC_W_AHEAD steps have been read); every
-    // step's activation registers are refilled with the same step of the following stage (`next_step` of `rows_next`)
-    auto stage = [&](int buffer, int next_step, const half2_t (&ratio)[2]) {
+    // step's activation register is refilled with the same step of the following stage (`next_step` of `rows_next`)
+    auto stage = [&](int buffer, int next_step, half2_t ratio) {
 #pragma unroll
         for (int s = 0; s < FSC_STEPS; ++s) {
             if (s + FSC_W_AHEAD < FSC_STEPS) {
                 read_step(buffer, s + FSC_W_AHEAD, w[(s + FSC_W_AHEAD) % RING]);
             }
+            const half8_t fragment = rescale(x[s], ratio);
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
-                const half8_t fragment = rescale(x[s][rt], ratio[rt]);
-#pragma unroll
-                for (int nt = 0; nt < FWD_NT; ++nt) {
-                    // (weights as the A operand: the lane ends up with one activation row and runs of four neighbouring
-                    // columns, which the epilogue stages with 8-byte LDS writes)
-                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[s % RING][nt], fragment, acc[rt][nt], 0, 0, 0);
-                }
+            for (int nt = 0; nt < FWD_NT; ++nt) {
+                // (weights as the A operand: the lane ends up with one activation row and runs of four neighbouring
+                // columns, which the epilogue stages with 8-byte LDS writes)
+                acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[s % RING][nt], fragment, acc[nt], 0, 0, 0);
             }
-            load_x(rows_next, next_step + s, x[s]);
+            x[s] = load_x(rows_next, next_step + s);
             // (the requests stay where they are written: moved to the end of the stage, as the scheduler would have
             // them, they leave the next stage waiting for memory)
             __builtin_amdgcn_sched_barrier(0);
@@ -674,23 +663,21 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
     FSC_LAP(1);
     read_first_steps(0);
     int item = 0, kb = 0;
+    float ratio_next = load_ratio(rows_next, 0);
 #pragma unroll 1
     for (int q = 0; q < total; ++q) {
         // (rows_next: still the rows of this super-block's item, whose stage 0 was requested with them)
-        uint4 sums[2] = {make_uint4(0, 0, 0, 0), make_uint4(0, 0, 0, 0)};
+        uint4 sums = make_uint4(0, 0, 0, 0);
         if constexpr (K45) {
-            load_sums(rows_next, kb, sums);
+            sums = load_sums(rows_next, kb);
         }
-        float ratio_f32[2];
-        load_ratio(rows_next, kb, ratio_f32);
-        {   // a 32-row tile without rows of the item multiplies zeros: no branch in the loop, and the matrix pipe draws
-            // less power on zeros, which the clock of the waves that do have rows gains from
-            const int wave_rows = item_field(item, 2) - item_field(item, 1) - wave * 64;
-            if (wave_rows <= 0) { ratio_f32[0] = 0.0f; }
-            if (wave_rows <= 32) { ratio_f32[1] = 0.0f; }
+        float ratio_f32 = ratio_next;   // (requested a stage ago: needed at once)
+        // a wave without rows in the item multiplies zeros: no branch in the loop, and the matrix pipe draws less
+        // power on zeros, which the clock of the waves that do have rows gains from
+        if (item_field(item, 1) + wave * 32 >= item_field(item, 2)) {
+            ratio_f32 = 0.0f;
         }
-        const half2_t ratio[2] = {half2_t{static_cast<_Float16>(ratio_f32[0]), static_cast<_Float16>(ratio_f32[0])},
-                                  half2_t{static_cast<_Float16>(ratio_f32[1]), static_cast<_Float16>(ratio_f32[1])}};
+        const half2_t ratio = {static_cast<_Float16>(ratio_f32), static_cast<_Float16>(ratio_f32)};
         // stage 0; requests stage 1 of the same super-block
         stage(0, kb * 16 + 8, ratio);
         FSC_LAP(2);
@@ -702,22 +689,18 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
         const int item_next = last_of_item ? min(item + 1, n_items - 1) : item;
         const int kb_next = last_of_item ? 0 : kb + 1;
         rows_next = rows_of(item_next);
+        ratio_next = load_ratio(rows_next, kb_next);
         stage(1, kb_next * 16, ratio);
         if constexpr (K45) {
             // the super-block's extra reduction step: block minima x block sums (slots 8..15 of the instruction are empty)
+            const half8_t block_sums = rescale(__builtin_bit_cast(half8_t, half != 0 ? make_uint4(0, 0, 0, 0) : sums), ratio);
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) {
                 uint4 minima = *reinterpret_cast<const uint4 *>(&lds.mins[q & 1][nt * 512 + l32 * 16]);
                 if (half != 0) {
                     minima = make_uint4(0, 0, 0, 0);
                 }
-#pragma unroll
-                for (int rt = 0; rt < 2; ++rt) {
-                    const uint4 block_sums = half != 0 ? make_uint4(0, 0, 0, 0) : sums[rt];
-                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, minima),
-                                                                         rescale(__builtin_bit_cast(half8_t, block_sums), ratio[rt]),
-                                                                         acc[rt][nt], 0, 0, 0);
-                }
+                acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, minima), block_sums, acc[nt], 0, 0, 0);
             }
         }
         FSC_LAP(4);
@@ -732,40 +715,35 @@ __global__ __launch_bounds__(FSC_THREADS, 2) void mmq_forward_scaled_kernel(cons
             const bool second = tile >= a.n_tiles;
             const int n0 = (second ? tile - a.n_tiles : tile) * FWD_TN;
             uint16_t * const y = second ? a.y_second : a.y;
-            const int wave_row = row_start + wave * 64;
+            const int r0 = row_start + wave * 32;
             // recomputing the lane's share here is cheaper than keeping it alive through the loop
             int lane_here = lane;
             asm volatile("" : "+v"(lane_here));
             const int l32_here = lane_here & 31, half_here = lane_here >> 5;
+            if (r0 < row_end) {
+                const float row_power = a.row_power[min(r0 + l32_here, a.rows_padded - 1)];
 #pragma unroll
-            for (int rt = 0; rt < 2; ++rt) {
-                const int r0 = wave_row + 32 * rt;
-                if (r0 < row_end) {
-                    const float row_power = a.row_power[min(r0 + l32_here, a.rows_padded - 1)];
+                for (int pair = 0; pair < 2; ++pair) {
 #pragma unroll
-                    for (int pair = 0; pair < 2; ++pair) {
+                    for (int t = 0; t < 2; ++t) {
+                        const int nt = 2 * pair + t;
 #pragma unroll
-                        for (int t = 0; t < 2; ++t) {
-                            const int nt = 2 * pair + t;
-#pragma unroll
-                            for (int j = 0; j < 4; ++j) {
-                                const float4 column_power =
-                                    *reinterpret_cast<const float4 *>(&lds.row_power[item & 1][nt * 32 + 8 * j + 4 * half_here]);
-                                acc[rt][nt][4 * j + 0] *= row_power * column_power.x;
-                                acc[rt][nt][4 * j + 1] *= row_power * column_power.y;
-                                acc[rt][nt][4 * j + 2] *= row_power * column_power.z;
-                                acc[rt][nt][4 * j + 3] *= row_power * column_power.w;
-                            }
+                        for (int j = 0; j < 4; ++j) {
+                            const float4 column_power =
+                                *reinterpret_cast<const float4 *>(&lds.row_power[item & 1][nt * 32 + 8 * j + 4 * half_here]);
+                            acc[nt][4 * j + 0] *= row_power * column_power.x;
+                            acc[nt][4 * j + 1] *= row_power * column_power.y;
+                            acc[nt][4 * j + 2] *= row_power * column_power.z;
+                            acc[nt][4 * j + 3] *= row_power * column_power.w;
                         }
-                        const v16f (&tiles)[2] = *reinterpret_cast<const v16f (*)[2]>(&acc[rt][2 * pair]);
-                        store_rows_32x64(lds.staging[wave], tiles,
-                                         y + static_cast<int64_t>(r0) * a.out_features + n0 + 64 * pair, a.out_features,
-                                         row_end - r0, a.out_features - n0 - 64 * pair, lane_here);
                     }
+                    const v16f (&tiles)[2] = *reinterpret_cast<const v16f (*)[2]>(&acc[2 * pair]);
+                    store_rows_32x64(lds.staging[wave], tiles, y + static_cast<int64_t>(r0) * a.out_features + n0 + 64 * pair,
+                                     a.out_features, row_end - r0, a.out_features - n0 - 64 * pair, lane_here);
                 }
-#pragma unroll
-                for (int nt = 0; nt < FWD_NT; ++nt) acc[rt][nt] = zero;
             }
+#pragma unroll
+            for (int nt = 0; nt < FWD_NT; ++nt) acc[nt] = zero;
             ++item;
             kb = 0;
             FSC_LAP(5);

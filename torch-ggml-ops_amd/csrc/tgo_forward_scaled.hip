@@ -120,7 +120,7 @@ constexpr int scale_offset() { return TYPE == Q3_K ? 108 : TYPE == Q6_K ? 208 : 
 __device__ unsigned long long fsc_times[8][2][96];
 // phase accumulators in scalar registers; nothing is stored before the end of the kernel
 #define FSC_LAP(slot) do { const unsigned long long now_ = __builtin_readcyclecounter(); lap[slot] += now_ - lap_last; lap_last = now_; } while (0)
-#define FSC_LAP_DUMP(role) do { if (profiled >= 0 && lane == 0) { for (int i_ = 0; i_ < 10; ++i_) fsc_times[profiled][role][i_ + 1] = lap[i_]; fsc_times[profiled][role][90] = n_items; fsc_times[profiled][role][94] = wall_clock64() - wall_start; } } while (0)
+#define FSC_LAP_DUMP(role) do { if (profiled >= 0 && lane == 0) { for (int i_ = 0; i_ < 10; ++i_) fsc_times[profiled][role][i_ + 1 + (wave == FSC_MULTIPLIERS - 1 ? 40 : 0)] = lap[i_]; fsc_times[profiled][role][90] = n_items; fsc_times[profiled][role][94] = wall_clock64() - wall_start; } } while (0)
 #else
 #define FSC_LAP(slot) do {} while (0)
 #define FSC_LAP_DUMP(role) do {} while (0)
@@ -213,7 +213,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         return;
     }
 #ifdef FSC_TIMING
-    const int profiled = (wave == 0 || wave == FSC_MULTIPLIERS) && blockIdx.x % 32 == 5 ? blockIdx.x / 32 : -1;
+    const int profiled = (wave == 0 || wave == FSC_MULTIPLIERS - 1 || wave == FSC_MULTIPLIERS) && blockIdx.x % 32 == 5 ? blockIdx.x / 32 : -1;
     unsigned long long lap[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     unsigned long long lap_last = __builtin_readcyclecounter();
     const unsigned long long wall_start = wall_clock64();
@@ -471,7 +471,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         };
 
 
-        // c_request walks RAW_DEPTH super-blocks ahead of c_park, which is one ahead of the super-block the
+        // c_request walks RAW_DEPTH super-blocks ahead of c_park, which is two ahead of the super-block the
         // multipliers work on; c_scan is the item whose scale words are in flight.
         Cursor c_request, c_park, c_scan;
         open_item(c_request, 0);
@@ -501,6 +501,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             step(c_request);
         };
         advance(0);
+        advance(1);
         StageInputs inputs = {};
         if constexpr (K45) {
             inputs = fetch_inputs(0, 0);
@@ -525,8 +526,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
                 unpack(std::integral_constant<int, 1>{}, parity, 1);
             }
             FSC_LAP(2);
-            advance(parity ^ 1);
-            FSC_LAP(3);
             if constexpr (K45) {
                 inputs = fetch_inputs(0, parity ^ 1);
             }
@@ -554,6 +553,10 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
                 unpack(std::integral_constant<int, 0>{}, parity ^ 1, 0);
             }
             FSC_LAP(6);
+            // slot `parity` is free (Q4_K/Q5_K: its last inputs are in registers; the others: stage 1 is done):
+            // super-block q + 2 goes there
+            advance(parity);
+            FSC_LAP(3);
             __syncthreads();
             FSC_LAP(4);
         }
@@ -625,7 +628,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     // weight fragments are read FSC_W_AHEAD reduction steps before their matrix instructions
     constexpr int RING = FSC_W_AHEAD + 1;
     half8_t w[RING][FWD_NT];
-    auto read_step = [&](int buffer, int step, half8_t (&out)[FWD_NT]) {
+    auto read_step = [&](int buffer, int step, half8_t (&out)[FWD_NT]) __attribute__((always_inline)) {
 #pragma unroll
         for (int nt = 0; nt < FWD_NT; ++nt) {
             out[nt] = *reinterpret_cast<const half8_t *>(&lds.wq[buffer][((nt * FSC_STEPS + step) * 64 + lane) * 16]);
@@ -633,13 +636,15 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     };
     // one stage: eight reduction steps from operand tile `buffer` (its first FSC_W_AHEAD steps have been read); every
     // step's activation register is refilled with the same step of the following stage (`next_step` of `rows_next`)
-    auto stage = [&](int buffer, int next_step, half2_t ratio) {
+    auto stage_as = [&](auto active_tag, int buffer, int next_step, half2_t ratio) __attribute__((always_inline)) {
+        constexpr bool ACTIVE = decltype(active_tag)::value;
 #pragma unroll
         for (int s = 0; s < FSC_STEPS; ++s) {
             if (s + FSC_W_AHEAD < FSC_STEPS) {
                 read_step(buffer, s + FSC_W_AHEAD, w[(s + FSC_W_AHEAD) % RING]);
             }
             const half8_t fragment = rescale(x[s], ratio);
+            if constexpr (ACTIVE)
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) {
                 // (weights as the A operand: the lane ends up with one activation row and runs of four neighbouring
@@ -650,6 +655,15 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             // (the requests stay where they are written: moved to the end of the stage, as the scheduler would have
             // them, they leave the next stage waiting for memory)
             __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    // (a wave without rows in the item keeps requesting activations, which may be the next item's, but leaves the matrix
+    // pipe to the wave it shares the SIMD with)
+    auto stage = [&](int buffer, int next_step, half2_t ratio, bool active) __attribute__((always_inline)) {
+        if (active) {
+            stage_as(std::true_type{}, buffer, next_step, ratio);
+        } else {
+            stage_as(std::false_type{}, buffer, next_step, ratio);
         }
     };
     auto read_first_steps = [&](int buffer) {
@@ -674,12 +688,10 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         float ratio_f32 = ratio_next;   // (requested a stage ago: needed at once)
         // a wave without rows in the item multiplies zeros: no branch in the loop, and the matrix pipe draws less
         // power on zeros, which the clock of the waves that do have rows gains from
-        if (item_field(item, 1) + wave * 32 >= item_field(item, 2)) {
-            ratio_f32 = 0.0f;
-        }
+        const bool active = item_field(item, 1) + wave * 32 < item_field(item, 2);
         const half2_t ratio = {static_cast<_Float16>(ratio_f32), static_cast<_Float16>(ratio_f32)};
         // stage 0; requests stage 1 of the same super-block
-        stage(0, kb * 16 + 8, ratio);
+        stage(0, kb * 16 + 8, ratio, active);
         FSC_LAP(2);
         __syncthreads();
         FSC_LAP(3);
@@ -690,10 +702,11 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         const int kb_next = last_of_item ? 0 : kb + 1;
         rows_next = rows_of(item_next);
         ratio_next = load_ratio(rows_next, kb_next);
-        stage(1, kb_next * 16, ratio);
+        stage(1, kb_next * 16, ratio, active);
         if constexpr (K45) {
             // the super-block's extra reduction step: block minima x block sums (slots 8..15 of the instruction are empty)
             const half8_t block_sums = rescale(__builtin_bit_cast(half8_t, half != 0 ? make_uint4(0, 0, 0, 0) : sums), ratio);
+            if (active)
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) {
                 uint4 minima = *reinterpret_cast<const uint4 *>(&lds.mins[q & 1][nt * 512 + l32 * 16]);

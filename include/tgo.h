@@ -48,9 +48,10 @@ int tgo_block_bytes(int quant_type);
 
 /* Bytes of the activation workspace the forward entry points need for `rows` rows of
  * `in_features` values: q8_1 blocks (two bytes per value, one fp32 scale and one fp32 sum per 32
- * values), rows padded to 32.  The arrangement inside is the library's business (32-row tiles in MFMA
- * fragment order holding the quants as fp16 numbers or as int8, see tgo_set_forward_operand, or plain
- * int8 rows for decode-sized calls); tgo_q8_workspace_unpack reads any of them.
+ * values, for the scaled operands also a power of two and 16 bytes of block sums per 256 values and a power of
+ * two per row), rows padded to 32.  The arrangement inside is the library's business (32-row tiles in MFMA
+ * fragment order holding the quants as int8, as fp16 numbers or as scaled fp16 values, see
+ * tgo_set_forward_operand, or plain int8 rows for decode-sized calls); tgo_q8_workspace_unpack reads any of them.
  * Replaces the workspace sizing in csrc/mmq_hip.cu:643-652 and :529-537. */
 int64_t tgo_q8_workspace_bytes(int64_t rows, int64_t in_features);
 
@@ -242,19 +243,33 @@ int tgo_profile_enable(int enabled);
 int tgo_profile_read(int kernel, double * total_ms, int64_t * launches);
 
 /* Matrix operands of the forward kernels that run on the matrix cores (not the decode-sized GEMV family), a
- * process-wide setting.  TGO_OPERAND_HALF multiplies fp16 numbers that hold the quantized activations and the
- * integer weight operands exactly, so the per-block dot products are the same integers as with int8 operands;
- * TGO_OPERAND_INT8 runs the int8 matrix instruction; TGO_OPERAND_AUTO (default) takes fp16 for IQ2_S (whose integer
- * operand needs two int8 planes but one fp16 number) and int8 for the other formats, and int8 for workspaces that
- * are quantized before their format is known (tgo_quantize_q8_1 / tgo_mmq_forward_prepared).  The activation workspace
- * is laid out for one of the two: do not change the setting between quantizing a workspace and using it.
- * tgo_forward_operand() returns the current setting.  No counterpart in the reference. */
+ * process-wide setting.
+ *   TGO_OPERAND_INT8    int8 quants on the int8 matrix instruction, scales applied per 32-value block in fp32 (the
+ *                       arithmetic of the reference's kernel, csrc/vendor/llama_cpp/mmq-vec-dot.cuh).
+ *   TGO_OPERAND_HALF    fp16 numbers that hold the quantized activations and the integer weight operands exactly:
+ *                       the same integer dot products per block as with int8 operands.
+ *   TGO_OPERAND_SCALED  both operands carry their scales into the matrix instruction: the dequantized q8_1
+ *                       activation and the dequantized weight, each normalised by a power of two per row and rounded
+ *                       to fp16 once (relative 2^-11; same quants, block scales and sums as the other kinds).  Results
+ *                       differ from the other kinds by up to 5e-4 of the largest output; the fastest kind for calls
+ *                       that fill the chip.  The fused SwiGLU entry point has no such kernel and takes int8 (fp16 for
+ *                       IQ2_S) when this kind is forced.
+ *   TGO_OPERAND_AUTO    (default) scaled for calls of at least 128 tiles of 256 rows x 128 outputs (total rows of
+ *                       a grouped call; both projections of a pair count), otherwise fp16 for IQ2_S (whose integer
+ *                       operand needs two int8 planes but one fp16 number) and int8 for the other formats.
+ * Workspaces that are quantized before their format is known (tgo_quantize_q8_1 / tgo_mmq_forward_prepared) take int8
+ * unless TGO_OPERAND_HALF is forced.  The activation workspace is laid out for one kind and says which in its last
+ * KiB: tgo_q8_workspace_unpack follows that tag, and tgo_mmq_forward_prepared turns its outputs into NaN when the
+ * setting was changed between quantizing a workspace and using it.  A call reads the setting once.
+ * tgo_forward_operand() returns the current setting; tgo_forward_operand_for() the kind (never AUTO) that a forward
+ * call of this format and shape would use under it (`projections`: 2 for a pair).  No counterpart in the reference. */
 #define TGO_OPERAND_INT8 0
 #define TGO_OPERAND_HALF 1
 #define TGO_OPERAND_AUTO 2
 #define TGO_OPERAND_SCALED 3
 int tgo_set_forward_operand(int operand);
 int tgo_forward_operand(void);
+int tgo_forward_operand_for(int quant_type, int64_t rows, int64_t out_features, int projections);
 
 #ifdef __cplusplus
 }

@@ -44,6 +44,22 @@ def assert_matches_f32_reference(actual_bf16: torch.Tensor, reference_f32: np.nd
     )
 
 
+# Noise allowance of assert_matches_f32_reference by operand kind of the forward kernel.  int8 and exact fp16 operands
+# compute the oracle's integer dot products and differ from it by fp32 summation order only.  The scaled kind rounds
+# every dequantized activation and weight to fp16 once (2^-11 relative each): with random signs the dot product's
+# error is a few 1e-4 of the largest output (measured: up to 2.9e-4 at K of 256 to 4096, up to 4.6e-4 for Q4_K/Q5_K at
+# 4096 rows, whose minimum term cancels a large part of the sum).
+OPERAND_NOISE = {"int8": 1e-4, "half": 1e-4, "scaled": 8e-4}
+
+
+def forward_noise(qtype: int, rows: int, out_features: int, projections: int = 1) -> float:
+    """Allowance for the kind the library uses for a forward call of this shape under the current setting (total rows
+    of a grouped call; projections: 2 for a pair)."""
+    from torch_ggml_ops import _native
+
+    return OPERAND_NOISE[_native.forward_operand_for(qtype, rows, out_features, projections)]
+
+
 def random_bf16(shape, seed, device="cuda", scale=1.0) -> torch.Tensor:
     generator = torch.Generator(device="cpu").manual_seed(seed)
     return (torch.randn(*shape, generator=generator) * scale).to(torch.bfloat16).to(device)

@@ -36,13 +36,20 @@ def test_library_exports_every_declared_symbol(package):
 def test_sizes_and_block_bytes(package):
     _, native, _, synth = package
     lib = native.lib
-    assert lib.tgo_version() >= 100
+    assert lib.tgo_version() >= 110   # (the workspace grew with the scaled operands: callers size it through the library)
     for qtype, size in synth.BLOCK_BYTES.items():
         assert lib.tgo_block_bytes(qtype) == size
     assert lib.tgo_block_bytes(10) == 0
-    # two bytes per value (the quants as fp16 numbers) + two fp32 per 32 values, rows padded to 32, plus the 1 KiB tail
-    assert lib.tgo_q8_workspace_bytes(33, 512) == 2 * 64 * 512 + 2 * 64 * 16 * 4 + 1024
+    # two bytes per value (fp16 operands) + two fp32 per 32 values + a power of two and 16 bytes of block sums per 256
+    # values + a power of two per row, rows padded to 32, plus the 1 KiB tail
+    assert lib.tgo_q8_workspace_bytes(33, 512) == 2 * 64 * 512 + 2 * 64 * 16 * 4 + 64 * 2 * (4 + 16) + 64 * 4 + 1024
     assert lib.tgo_q8_workspace_bytes(0, 512) == 0
+    # the kind a call would use: scaled once it has 128 tiles of 256 rows x 128 outputs (both projections count)
+    assert native.forward_operand() == "auto"
+    assert native.forward_operand_for(13, 4096, 1024, 1) == "scaled"
+    assert native.forward_operand_for(13, 4096, 1024 - 128, 1) == "int8"
+    assert native.forward_operand_for(22, 512, 4096, 1) == "half"
+    assert native.forward_operand_for(22, 2048, 1024, 2) == "scaled"
     assert lib.tgo_task_workspace_bytes(100, 7) % 16 == 0
     assert lib.tgo_task_workspace_bytes(100, 7) >= 4 * (1 + 3 * (13 + 7))
 

@@ -17,7 +17,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import QTYPES, assert_matches_f32_reference, bits, f32, max_rel_to_peak, nrmse
+from helpers import QTYPES, assert_matches_f32_reference, bits, f32, forward_noise, max_rel_to_peak, nrmse
 
 pytestmark = pytest.mark.gpu
 
@@ -62,7 +62,7 @@ def _check_forward(tgo, oracle, qtype, x, packed_host, packed, n, rows):
     index = torch.tensor(rows, device="cuda")
     x_rows = bits(x.index_select(0, index))
     picked = out.index_select(0, index)
-    assert_matches_f32_reference(picked, oracle.mmq_forward(qtype, x_rows, packed_host, n, K))
+    assert_matches_f32_reference(picked, oracle.mmq_forward(qtype, x_rows, packed_host, n, K), forward_noise(qtype, x.shape[0], n))
     expected = oracle.linear_forward(qtype, x_rows, packed_host, n, K)
     assert nrmse(f32(picked), expected) < FORWARD_TOLERANCE
     assert max_rel_to_peak(f32(picked), expected) < FORWARD_TOLERANCE

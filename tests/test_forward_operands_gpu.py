@@ -1,17 +1,18 @@
-"""The forward kernels under both kinds of matrix operand (run with -m gpu).
+"""The forward kernels under every kind of matrix operand (run with -m gpu).
 
-The library multiplies either int8 values or fp16 numbers that hold the same integers exactly
-(`tgo_set_forward_operand`); by default the format decides.  Every check here runs once with each kind
-forced, for all five formats: the quantizer's workspace against the oracle bit for bit, dense, grouped,
-pair and fused-SwiGLU results against the oracle's forward algebra, dense == grouped bit for bit, and the
-two kinds against each other (same integers, different order of the fp32 scale products).
+The library multiplies int8 values, fp16 numbers that hold the same integers exactly, or fp16 numbers that
+carry the scales as well (`tgo_set_forward_operand`); by default the format and the size of the call decide.
+Every check here runs once with each kind forced, for all five formats: the quantizer's workspace against
+the oracle bit for bit, dense, grouped, pair and fused-SwiGLU results against the oracle's forward algebra,
+dense == grouped bit for bit, and the kinds against each other (int8 and exact fp16: same integers, different
+order of the fp32 scale products; scaled: two fp16 roundings per product on top).
 """
 
 import numpy as np
 import pytest
 import torch
 
-from helpers import QTYPES, assert_matches_f32_reference, bits, f32, max_rel_to_peak, nrmse, random_bf16
+from helpers import OPERAND_NOISE, QTYPES, assert_matches_f32_reference, bits, f32, max_rel_to_peak, nrmse, random_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -27,7 +28,7 @@ def ops():
     return torch_ggml_ops, _native, synth
 
 
-@pytest.fixture(params=("int8", "half"))
+@pytest.fixture(params=("int8", "half", "scaled"))
 def operand(request, ops):
     _, native, _ = ops
     native.set_forward_operand(request.param)
@@ -53,7 +54,8 @@ def test_setting_is_validated_and_defaults_to_auto(ops):
 
 @pytest.mark.parametrize("rows,k", [(33, 512), (129, 2048)])
 def test_workspace_holds_the_oracle_quants(ops, oracle, operand, rows, k):
-    """The format-less quantizer entry follows a forced setting; its fp16 tiles unpack to the same int8 values."""
+    """The format-less quantizer entry follows a forced exact kind (int8 when the scaled kind is forced); its fp16
+    tiles unpack to the same int8 values."""
     _, native, _ = ops
     x = random_bf16((rows, k), seed=70 + rows, scale=2.0)
     x[0, :32] = 0
@@ -82,7 +84,7 @@ def test_dense_forward_matches_oracle(ops, oracle, operand, qname, rows, n, k):
     x = random_bf16((rows, k), seed=rows + k)
     actual = tgo.mmq(x, host.cuda(), qtype, n)
     assert torch.isfinite(actual).all()
-    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k))
+    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k), OPERAND_NOISE[operand])
     expected = oracle.linear_forward(qtype, bits(x), host.numpy(), n, k)
     assert nrmse(f32(actual), expected) < FORWARD_TOLERANCE
     assert max_rel_to_peak(f32(actual), expected) < FORWARD_TOLERANCE
@@ -106,7 +108,7 @@ def test_extreme_blocks_stay_exact(ops, oracle, operand, qname):
     signs = torch.from_numpy(rng.choice(np.array([-1.0, 1.0], dtype=np.float32), size=(rows, k)))
     x = (signs * 3.0).to(torch.bfloat16).cuda()
     actual = tgo.mmq(x, host.cuda(), qtype, n)
-    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k))
+    assert_matches_f32_reference(actual, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k), OPERAND_NOISE[operand])
 
 
 @pytest.mark.parametrize("qname", tuple(QTYPES))
@@ -122,7 +124,7 @@ def test_grouped_forward_matches_oracle_and_dense(ops, oracle, operand, qname):
     x = random_bf16((offsets[-1], k), seed=4321)
     actual = tgo.grouped_mmq(x, device, *_metadata(experts, offsets), qtype, n)
     exact = oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n)
-    assert_matches_f32_reference(actual, exact)
+    assert_matches_f32_reference(actual, exact, OPERAND_NOISE[operand])
     begin = 0
     for expert, end in zip(experts, offsets):
         if end - begin > 32:   # (up to 32 rows a dense call takes the GEMV family, another summation order)
@@ -146,8 +148,8 @@ def test_pair_and_fused_swiglu(ops, oracle, operand, qname):
     torch.testing.assert_close(up, tgo.grouped_mmq(x, up_host.cuda(), *metadata, qtype, n), rtol=0, atol=0)
     gate_ref = oracle.grouped(oracle.mmq_forward, qtype, bits(x), gate_host.numpy(), experts, offsets, n, k, n)
     up_ref = oracle.grouped(oracle.mmq_forward, qtype, bits(x), up_host.numpy(), experts, offsets, n, k, n)
-    assert_matches_f32_reference(gate, gate_ref)
-    assert_matches_f32_reference(up, up_ref)
+    assert_matches_f32_reference(gate, gate_ref, OPERAND_NOISE[operand])
+    assert_matches_f32_reference(up, up_ref, OPERAND_NOISE[operand])
     activated = tgo.grouped_mmq_swiglu(x, gate_host.cuda(), up_host.cuda(), *metadata, qtype, n)
     gate_bf16 = torch.from_numpy(gate_ref).to(torch.bfloat16).double().numpy()
     with np.errstate(over="ignore"):
@@ -157,23 +159,77 @@ def test_pair_and_fused_swiglu(ops, oracle, operand, qname):
 
 
 @pytest.mark.parametrize("qname", tuple(QTYPES))
-def test_both_kinds_agree(ops, qname):
-    """Same integer dot products, fp32 scale products in a different order: the results differ by fp32 rounding
-    before the final bf16 rounding, i.e. at most one bf16 ulp here and there."""
+def test_kinds_agree(ops, qname):
+    """int8 against exact fp16: same integer dot products, fp32 scale products in a different order, so the results
+    differ by fp32 rounding before the final bf16 rounding, i.e. at most one bf16 ulp here and there.  The scaled
+    kind adds two fp16 roundings per product.  A small call under "auto" takes the exact kind of its format."""
     tgo, native, synth = ops
     qtype, rows, n, k = QTYPES[qname], 300, 256, 2048
     weight = synth.random_packed_weight(qtype, (n,), k, seed=800 + qtype).cuda()
     x = random_bf16((rows, k), seed=55)
     results = {}
     try:
-        for kind in ("int8", "half"):
+        for kind in ("int8", "half", "scaled"):
             native.set_forward_operand(kind)
             results[kind] = f32(tgo.mmq(x, weight, qtype, n)).astype(np.float64)
     finally:
         native.set_forward_operand("auto")
+    peak = np.abs(results["int8"]).max()
     difference = np.abs(results["int8"] - results["half"])
-    assert (difference <= np.abs(results["int8"]) * 2.0**-7 + 1e-6 * np.abs(results["int8"]).max()).all()
+    assert (difference <= np.abs(results["int8"]) * 2.0**-7 + 1e-6 * peak).all()
     assert nrmse(results["half"], results["int8"]) < 1e-3
-    native.set_forward_operand("auto")
+    difference = np.abs(results["int8"] - results["scaled"])
+    assert (difference <= np.abs(results["int8"]) * 2.0**-7 + OPERAND_NOISE["scaled"] * peak).all()
+    assert nrmse(results["scaled"], results["int8"]) < 2e-3
+    assert native.forward_operand_for(qtype, rows, n) == ("half" if qname == "IQ2_S" else "int8")
     chosen = f32(tgo.mmq(x, weight, qtype, n)).astype(np.float64)
     np.testing.assert_array_equal(chosen, results["half" if qname == "IQ2_S" else "int8"])
+
+
+@pytest.mark.parametrize("qname", ("IQ2_S", "Q5_K"))
+@pytest.mark.parametrize("rows,n", [(300, 256), (2048, 2048)])
+def test_workspace_of_a_forward_call_unpacks_by_its_tag(ops, oracle, qname, rows, n):
+    """Under "auto" the kind depends on the call (here: exact fp16 or int8 for the small one, scaled for the large
+    one), so whoever reads the workspace afterwards cannot derive its layout from the setting: the unpacker follows
+    the tag that the quantizer left in the workspace.  All layouts give back the oracle's quants, scales and sums."""
+    _, native, synth = ops
+    qtype, k = QTYPES[qname], 512
+    assert native.forward_operand() == "auto"
+    assert native.forward_operand_for(qtype, rows, n) == ("scaled" if rows == 2048 else "half" if qname == "IQ2_S" else "int8")
+    weight = synth.random_packed_weight(qtype, (n,), k, seed=900 + qtype).cuda()
+    x = random_bf16((rows, k), seed=91, scale=2.0)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    workspace = torch.empty(native.lib.tgo_q8_workspace_bytes(rows, k), dtype=torch.uint8, device="cuda")
+    native.check(native.lib.tgo_mmq_forward(x.data_ptr(), weight.data_ptr(), out.data_ptr(), workspace.data_ptr(), rows, k, n, qtype, None))
+    q = torch.empty(rows, k, dtype=torch.int8, device="cuda")
+    d = torch.empty(rows, k // 32, dtype=torch.float32, device="cuda")
+    s = torch.empty(rows, k // 32, dtype=torch.float32, device="cuda")
+    native.check(native.lib.tgo_q8_workspace_unpack(workspace.data_ptr(), q.data_ptr(), d.data_ptr(), s.data_ptr(), rows, k, None))
+    torch.cuda.synchronize()
+    q_ref, d_ref, s_ref = oracle.quantize_q8_1(bits(x))
+    np.testing.assert_array_equal(q.cpu().numpy(), q_ref)
+    np.testing.assert_array_equal(d.cpu().numpy().view(np.uint32), d_ref.view(np.uint32))
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+
+
+def test_prepared_forward_refuses_a_workspace_of_another_kind(ops):
+    """A workspace quantized under one forced kind and multiplied under another: every output is NaN."""
+    tgo, native, synth = ops
+    qtype, rows, n, k = QTYPES["Q4_K"], 64, 64, 512
+    weight = synth.random_packed_weight(qtype, (n,), k, seed=77).cuda()
+    x = random_bf16((rows, k), seed=3)
+    workspace = torch.empty(native.lib.tgo_q8_workspace_bytes(rows, k), dtype=torch.uint8, device="cuda")
+    out = torch.zeros(rows, n, dtype=torch.bfloat16, device="cuda")
+    try:
+        native.set_forward_operand("half")
+        native.check(native.lib.tgo_quantize_q8_1(x.data_ptr(), workspace.data_ptr(), rows, k, None))
+        native.check(native.lib.tgo_mmq_forward_prepared(workspace.data_ptr(), weight.data_ptr(), out.data_ptr(), rows, k, n, qtype, None))
+        torch.cuda.synchronize()
+        assert torch.isfinite(out).all()
+        torch.testing.assert_close(out, tgo.mmq(x, weight, qtype, n), rtol=0, atol=0)
+        native.set_forward_operand("int8")
+        native.check(native.lib.tgo_mmq_forward_prepared(workspace.data_ptr(), weight.data_ptr(), out.data_ptr(), rows, k, n, qtype, None))
+        torch.cuda.synchronize()
+        assert torch.isnan(out).all()
+    finally:
+        native.set_forward_operand("auto")

@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import QTYPES, assert_matches_f32_reference, bits
+from helpers import QTYPES, assert_matches_f32_reference, bits, forward_noise
 
 pytestmark = pytest.mark.gpu
 
@@ -93,14 +93,15 @@ def test_pair_forward_and_backward_at_the_benchmark_size(ops, oracle):
     sample = _sample_rows(offsets.cpu().numpy(), rng)
     expert_of_group = indices.cpu().numpy()
     gate_host, up_host = {}, {}
+    noise = forward_noise(qtype, x.shape[0], n, 2)
     for group, row in sample:
         expert = int(expert_of_group[group])
         if expert not in gate_host:
             gate_host[expert] = gate[expert].cpu().numpy()
             up_host[expert] = up[expert].cpu().numpy()
         x_row = bits(x[row:row + 1])
-        assert_matches_f32_reference(out_gate[row:row + 1], oracle.mmq_forward(qtype, x_row, gate_host[expert], n, k))
-        assert_matches_f32_reference(out_up[row:row + 1], oracle.mmq_forward(qtype, x_row, up_host[expert], n, k))
+        assert_matches_f32_reference(out_gate[row:row + 1], oracle.mmq_forward(qtype, x_row, gate_host[expert], n, k), noise)
+        assert_matches_f32_reference(out_up[row:row + 1], oracle.mmq_forward(qtype, x_row, up_host[expert], n, k), noise)
         expected = oracle.grad_input(qtype, bits(grad_gate[row:row + 1]), gate_host[expert], n, k).astype(np.float64)
         expected += oracle.grad_input(qtype, bits(grad_up[row:row + 1]), up_host[expert], n, k)
         assert_matches_f32_reference(pair_grad[row:row + 1], expected.astype(np.float32), accumulate_noise=2e-6)
@@ -123,7 +124,7 @@ def test_down_projection_at_its_configured_size(ops, oracle):
     expert_of_group = indices.cpu().numpy()
     for group, row in _sample_rows(offsets.cpu().numpy(), np.random.default_rng(4), per_kind=4):
         host = down[int(expert_of_group[group])].cpu().numpy()
-        assert_matches_f32_reference(out[row:row + 1], oracle.mmq_forward(qtype, bits(x[row:row + 1]), host, n, k))
+        assert_matches_f32_reference(out[row:row + 1], oracle.mmq_forward(qtype, bits(x[row:row + 1]), host, n, k), forward_noise(qtype, x.shape[0], n))
 
 
 @pytest.mark.parametrize("qname", tuple(QTYPES))
@@ -142,7 +143,8 @@ def test_dense_at_its_largest_configured_size(ops, oracle, qname):
     torch.testing.assert_close(torch.ops.torch_ggml_ops.mmq_grad_input.default(dy * 2, weight, qtype, k), grad * 2, rtol=0, atol=0)
     rows = torch.tensor([0, 1, 127, 128, 255, 256, 2049, 4095], device="cuda")
     packed = host.numpy()
-    assert_matches_f32_reference(out.index_select(0, rows), oracle.mmq_forward(qtype, bits(x.index_select(0, rows)), packed, n, k))
+    assert_matches_f32_reference(out.index_select(0, rows), oracle.mmq_forward(qtype, bits(x.index_select(0, rows)), packed, n, k),
+                                 forward_noise(qtype, x.shape[0], n))
     assert_matches_f32_reference(
         grad.index_select(0, rows), oracle.grad_input(qtype, bits(dy.index_select(0, rows)), packed, n, k),
         accumulate_noise=2e-6,

@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import QTYPES, assert_matches_f32_reference, bits, f32, max_rel_to_peak, nrmse, random_bf16
+from helpers import QTYPES, assert_matches_f32_reference, bits, f32, forward_noise, max_rel_to_peak, nrmse, random_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -258,7 +258,8 @@ def test_more_groups_than_one_listing_pass(ops, oracle, qname):
     host, device = _experts(synth, qtype, 700, n, k, seed=380 + qtype)
     x = random_bf16((rows, k), seed=1212)
     actual = tgo.grouped_mmq(x, device, *_metadata(experts, offsets), qtype, n)
-    assert_matches_f32_reference(actual, oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n))
+    assert_matches_f32_reference(actual, oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n),
+                                 forward_noise(qtype, x.shape[0], n))
     grad = random_bf16((rows, n), seed=1313)
     actual = torch.ops.torch_ggml_ops.grouped_mmq_grad_input.default(grad, device, *_metadata(experts, offsets), qtype, k)
     expected = oracle.grouped(oracle.grad_input, qtype, bits(grad), host.numpy(), experts, offsets, n, k, k)

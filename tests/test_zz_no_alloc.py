@@ -64,3 +64,23 @@ def test_static_workspace_rejects_what_does_not_fit(native):
     assert lib.tgo_q8_workspace_bytes(rows, k) > 4 * 1024 * 1024
     assert lib.tgo_mmq_forward_static(p, p, p, rows, k, 8, 12, None) == 1
     assert b"static workspace" in lib.tgo_last_error()
+
+
+def test_static_workspace_forward_leaves_device_memory_alone(native):
+    """The driver's count of free device memory is the same before and after calls of the static form (inputs and
+    outputs allocated beforehand; the first call, which looks up the array's address, comes before the count)."""
+    _native, synth = native
+    lib = _native.lib
+    qtype, rows, n, k = QTYPES["Q5_K"], 300, 200, 1024
+    packed = synth.random_packed_weight(qtype, (n,), k, seed=7).cuda()
+    x = torch.randn(rows, k, device="cuda").to(torch.bfloat16)
+    out = torch.empty(rows, n, dtype=torch.bfloat16, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    _native.check(lib.tgo_mmq_forward_static(x.data_ptr(), packed.data_ptr(), out.data_ptr(), rows, k, n, qtype, stream))
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for smaller in (rows, 77, 1):
+        _native.check(lib.tgo_mmq_forward_static(x.data_ptr(), packed.data_ptr(), out.data_ptr(), smaller, k, n, qtype, stream))
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before

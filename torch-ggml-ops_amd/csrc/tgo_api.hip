@@ -190,7 +190,7 @@ ProfileScope::~ProfileScope() {
 
 extern "C" {
 
-int tgo_version(void) { return 100; }
+int tgo_version(void) { return 110; }
 
 int tgo_profile_enable(int enabled) {
     std::lock_guard<std::mutex> lock(g_profile_mutex);
@@ -210,6 +210,10 @@ int tgo_set_forward_operand(int operand) {
 }
 
 int tgo_forward_operand(void) { return tgo::forward_operand_setting(); }
+
+int tgo_forward_operand_for(int quant_type, int64_t rows, int64_t out_features, int projections) {
+    return tgo::forward_operand_kind(quant_type, rows, out_features, projections);
+}
 
 int tgo_profile_read(int kernel, double * total_ms, int64_t * launches) {
     if (kernel < 0 || kernel >= TGO_KERNEL_COUNT || total_ms == nullptr || launches == nullptr) {
@@ -312,7 +316,8 @@ int tgo_mmq_forward(const void * input_bf16, const void * packed, void * output_
     TGO_TRY(check_pointer(output_bf16, "output"));
     TGO_TRY(check_pointer(workspace, "workspace"));
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
-    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(quant_type));
+    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0),
+                                                         tgo::forward_operand_kind(quant_type, rows, out_features, 1));
     TGO_TRY(check_hip(tgo::launch_quantize_q8_1(static_cast<const uint16_t *>(input_bf16), view, rows, in_features,
                                                 hip_stream),
                       "quantize_q8_1 launch"));
@@ -352,11 +357,16 @@ int tgo_mmq_forward_prepared(const void * workspace, const void * packed, void *
     const tgo::Q8Workspace view =
         tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(0));
     const auto launch = tgo::use_gemv(rows, 0) ? tgo::launch_mmq_gemv : tgo::launch_mmq_forward;
-    return check_hip(launch(static_cast<const uint8_t *>(packed), nullptr, 0, view,
-                            static_cast<uint16_t *>(output_bf16), nullptr, nullptr, static_cast<int>(rows),
-                            static_cast<int>(in_features), static_cast<int>(out_features), quant_type,
-                            static_cast<hipStream_t>(stream)),
-                     "mmq_forward_prepared launch");
+    TGO_TRY(check_hip(launch(static_cast<const uint8_t *>(packed), nullptr, 0, view,
+                             static_cast<uint16_t *>(output_bf16), nullptr, nullptr, static_cast<int>(rows),
+                             static_cast<int>(in_features), static_cast<int>(out_features), quant_type,
+                             static_cast<hipStream_t>(stream)),
+                      "mmq_forward_prepared launch"));
+    // (the workspace was quantized by an earlier call: had the operand setting changed in between, its layout would
+    // not be the one this launch assumed)
+    return check_hip(tgo::launch_workspace_guard(view, static_cast<uint16_t *>(output_bf16), rows * out_features,
+                                                 static_cast<hipStream_t>(stream)),
+                     "workspace guard launch");
 }
 
 int tgo_mmq_grad_input(const void * grad_output_bf16, const void * packed, void * grad_input_bf16,
@@ -409,7 +419,7 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
     // (the fused SwiGLU epilogue exists in the MFMA kernel only)
     const bool gemv = !swiglu && tgo::use_gemv(rows, num_groups);
     // (the scaled-operand kernel has no fused SwiGLU epilogue)
-    int operand_kind = tgo::forward_operand_kind(quant_type);
+    int operand_kind = tgo::forward_operand_kind(quant_type, rows, out_features, packed_second != nullptr ? 2 : 1);
     if (swiglu && operand_kind == tgo::OPERAND_SCALED) {
         operand_kind = quant_type == TGO_TYPE_IQ2_S ? tgo::OPERAND_HALF : tgo::OPERAND_INT8;
     }

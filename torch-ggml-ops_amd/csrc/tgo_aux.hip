@@ -1,5 +1,6 @@
 // Auxiliary gfx950 kernels: weight dequantizer, q8_1 activation quantizer (which also builds the tile-task list
 // of a grouped call on the side), workspace inspection and the routing-weighted row -> token combine.
+#include <atomic>
 #include "tgo_device.h"
 #include "tgo_launch.h"
 
@@ -62,9 +63,9 @@ hipError_t launch_dequant_bf16(const uint8_t * packed, uint16_t * out, int64_t r
 }
 
 // ---- matrix operands of the forward kernels (process-wide) -------------------------------------------
-static int g_forward_operand = OPERAND_AUTO;
-int forward_operand_setting() { return g_forward_operand; }
-void set_forward_operand_setting(int operand) { g_forward_operand = operand; }
+static std::atomic<int> g_forward_operand{OPERAND_AUTO};
+int forward_operand_setting() { return g_forward_operand.load(std::memory_order_relaxed); }
+void set_forward_operand_setting(int operand) { g_forward_operand.store(operand, std::memory_order_relaxed); }
 
 // ---- bf16 activations -> q8_1 -------------------------------------------------------------------
 // Arithmetic of the reference quantizer (csrc/mmq_core.cuh:151-209): per 32 values amax, d = amax/127,
@@ -519,6 +520,29 @@ hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float
     const int64_t total = rows * in_features;
     q8_unpack_kernel<<<static_cast<unsigned>((total + 255) / 256), 256, 0, stream>>>(
         ws.q, ws.d, ws.sum, ws.power, ws.row_power, ws.tag, q, d, sum, static_cast<int>(rows), static_cast<int>(in_features));
+    return hipGetLastError();
+}
+
+// ---- a prepared workspace consumed as the wrong kind ---------------------------------------------------------
+// The quantizer and a later tgo_mmq_forward_prepared each derive the workspace layout from the process-wide operand
+// setting; a change of the setting between the two would make the multiply kernel read the bytes as another layout.
+// The host cannot see the tag without a synchronisation, so this runs behind the multiply kernel: when the tag is not
+// the one the launch assumed, every output becomes NaN (bf16 0x7fc0) instead of plausible garbage.  With the right
+// tag each thread reads one word and leaves.
+__global__ __launch_bounds__(256) void workspace_guard_kernel(const uint32_t * __restrict__ tag, uint32_t expected,
+                                                              uint16_t * __restrict__ out, int64_t count) {
+    if (*tag == expected) {
+        return;
+    }
+    for (int64_t i = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x; i < count; i += static_cast<int64_t>(gridDim.x) * 256) {
+        out[i] = 0x7fc0u;
+    }
+}
+
+hipError_t launch_workspace_guard(const Q8Workspace & ws, uint16_t * out, int64_t count, hipStream_t stream) {
+    const unsigned grid = static_cast<unsigned>(count < 256 * 1024 ? (count + 255) / 256 : 1024);
+    workspace_guard_kernel<<<grid == 0 ? 1 : grid, 256, 0, stream>>>(ws.tag, WORKSPACE_TAG_MAGIC | static_cast<uint32_t>(ws.layout),
+                                                                     out, count);
     return hipGetLastError();
 }
 

@@ -24,8 +24,13 @@
 // their fp16 operand tile (packed blocks RAW_DEPTH super-blocks ahead in registers, parked in the wave's own LDS
 // slot; LDS executes a wave's accesses in order, so these steps need no workgroup barrier).  Each SIMD then holds two
 // waves that feed the matrix pipe and one that keeps the vector pipe busy.  A super-block is two stages of 128
-// values; the operand tile of a stage (32 KiB, fragment order) is double buffered and one barrier per stage hands
-// it over: while the multipliers work on stage g, the unpackers write stage g + 1.
+// values; the operand tile of a stage (32 KiB, fragment order) goes through a ring of three buffers.  No workgroup
+// barrier hands a buffer over: every unpacking wave counts the stages it has written and every multiplying wave the
+// stages it has read, in LDS; a multiplier starts stage g when all four unpackers have counted g + 1, an unpacker
+// overwrites the buffer of stage g - 3 when all eight multipliers have counted g - 2.  (A barrier per stage makes
+// every stage as long as its slowest wave: twelve waves with memory latencies of their own then wait a quarter of
+// the time.)  LDS executes a wave's accesses in issue order, so a counter written after the data, or after the
+// last read, needs no wait of its own.
 //
 // A workgroup is persistent: it owns every gridDim.x-th (task, column tile) item of the launch and runs their
 // super-blocks as one stream, so an item's first loads (task description, packed blocks, the scan of its scales,
@@ -48,19 +53,14 @@ constexpr int FSC_STEPS = 8;                                // 16-value reductio
 constexpr int FSC_TILE_BYTES = FWD_NT * FSC_STEPS * 1024;   // fp16 operand of a stage: [tile][step][64 lanes][16 bytes]
 constexpr int FSC_ROWS = 256;                               // activation rows per task
 static_assert(FSC_ROWS == forward_row_tile(12, OPERAND_SCALED), "task rows match the workgroup");
-#ifndef FSC_TOUCH_AHEAD
-#define FSC_TOUCH_AHEAD 4
-#endif
 #ifndef FSC_W_AHEAD
 #define FSC_W_AHEAD 1
-#endif
-#ifndef FSC_X_AHEAD
-#define FSC_X_AHEAD 8
 #endif
 
 constexpr int FSC_MAX_ITEMS = 64;      // items per workgroup (one wave builds the table)
 constexpr int FSC_GRID = 256;          // one workgroup per CU
-constexpr int FSC_STAGE_PITCH = 68;    // bf16 per staged row: 64 columns + padding (34 words: 32 rows on 32 different banks)
+constexpr int FSC_BUFFERS = 3;         // operand tiles in flight between the unpacking and the multiplying waves
+constexpr int FSC_SPIN_LIMIT = 1 << 20;   // polls of a stage counter before a wave gives up waiting (a few hundred ms)
 
 struct ScaledItem {
     int expert, row_start, row_end, tile;   // tile: column tile + n_tiles * projection
@@ -74,11 +74,15 @@ struct ScaledLds {
     static constexpr int RAW_SLOT = K45 ? Format<TYPE>::BLOCK_BYTES
                                         : (Format<TYPE>::RAW_PITCH > WideStage<TYPE>::PITCH ? Format<TYPE>::RAW_PITCH
                                                                                              : WideStage<TYPE>::PITCH);
-    alignas(16) uint8_t wq[2][FSC_TILE_BYTES];                 // operand tiles of two stages
+    alignas(16) uint8_t wq[FSC_BUFFERS][FSC_TILE_BYTES];       // ring of operand tiles, one stage each
     alignas(16) uint8_t raw[4][2][32 * RAW_SLOT];              // per unpacking wave: packed blocks of two super-blocks
-    alignas(16) uint8_t mins[2][K45 ? FWD_NT * 512 : 16];      // fp16(-dmin * m * 2^-S): [tile][32 rows][8 blocks], by parity
-    alignas(16) float row_power[2][FWD_TN];                    // 2^S of the tile's weight rows, by the item's parity
-    alignas(16) uint16_t staging[FSC_MULTIPLIERS][32 * FSC_STAGE_PITCH];   // per multiplying wave: 32 rows x 64 columns of results
+    // fp16(-dmin * m * 2^-S): [tile][32 rows][8 blocks], beside the operand tile of the super-block's first stage
+    alignas(16) uint8_t mins[FSC_BUFFERS][K45 ? FWD_NT * 512 : 16];
+    // 2^S of the tile's weight rows by item & 3 (the unpackers open at most the second item after the one whose
+    // results are being stored)
+    alignas(16) float row_power[4][FWD_TN];
+    alignas(16) int produced[4];                               // stages written, per unpacking wave
+    alignas(16) int consumed[FSC_MULTIPLIERS];                 // stages read, per multiplying wave
     ScaledItem items[FSC_MAX_ITEMS];
     int item_count;
     std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;
@@ -126,48 +130,46 @@ __device__ unsigned long long fsc_times[8][2][96];
 #define FSC_LAP_DUMP(role) do {} while (0)
 #endif
 
-// Stores a 32-row x 64-column block of results that the matrix instructions left transposed (weights as the A
-// operand: the lane holds row l32 and, as element v of tile t, column 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4) as
-// bf16 rows: the wave transposes through `stage` (32 x FSC_STAGE_PITCH bf16 that only this wave touches) and every
-// lane stores 16-byte pieces, whole 128-byte rows.  `dst` points at row 0, column 0; rows >= valid_rows and columns >=
-// valid_cols are skipped.  The 16-byte path needs row_stride % 8 == 0 (dst is then 16-byte aligned: the tensor is,
-// and column tiles start at multiples of 64).
-TGO_DEVICE void store_rows_32x64(uint16_t * stage, const v16f (&tiles)[2], uint16_t * dst, int64_t row_stride,
-                                 int valid_rows, int valid_cols, int lane) {
+// Stores the wave's 32 rows x 128 columns of results, which the matrix instructions left transposed (weights as the
+// A operand: the lane holds row l32 and, as element v of tile t, column 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4), as
+// bf16.  The two half-waves exchange runs of four columns, after which a lane holds eight neighbouring columns and
+// stores 16 bytes; a row gets 32 contiguous bytes per instruction.  `dst` points at row 0, column 0; rows >=
+// valid_rows and columns >= valid_cols are skipped.  The 16-byte path needs row_stride % 8 == 0 (dst is then 16-byte
+// aligned: the tensor is, and column tiles start at multiples of 128).
+TGO_DEVICE void store_rows_32x128(const v16f (&tiles)[FWD_NT], uint16_t * dst, int64_t row_stride, int valid_rows,
+                                  int valid_cols, int lane) {
     const int l32 = lane & 31;
     const int half = lane >> 5;
-#pragma unroll
-    for (int t = 0; t < 2; ++t) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            *reinterpret_cast<uint2 *>(&stage[l32 * FSC_STAGE_PITCH + t * 32 + 8 * j + 4 * half]) =
-                make_uint2(pack_bf16x2(tiles[t][4 * j], tiles[t][4 * j + 1]), pack_bf16x2(tiles[t][4 * j + 2], tiles[t][4 * j + 3]));
-        }
-    }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
     const bool wide = (row_stride & 7) == 0;
+    uint16_t * const row = dst + l32 * row_stride;
 #pragma unroll
-    for (int p = 0; p < 4; ++p) {
-        const int id = lane + 64 * p;
-        const int r = id >> 3;
-        const int c = (id & 7) * 8;
-        if (r < valid_rows && c < valid_cols) {
-            const uint16_t * values = &stage[r * FSC_STAGE_PITCH + c];
-            if (wide && c + 8 <= valid_cols) {
-                // (rows of the staging area start 8-byte aligned: two 8-byte reads)
-                const uint2 low = *reinterpret_cast<const uint2 *>(values);
-                const uint2 high = *reinterpret_cast<const uint2 *>(values + 4);
-                *reinterpret_cast<uint4 *>(dst + r * row_stride + c) = make_uint4(low.x, low.y, high.x, high.y);
-            } else {
-                for (int e = 0; e < 8 && c + e < valid_cols; ++e) {
-                    dst[r * row_stride + c + e] = values[e];
+    for (int t = 0; t < FWD_NT; ++t) {
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            // runs 2m and 2m + 1 of the tile: the lower half-wave keeps its run 2m and takes the upper one's,
+            // the upper half-wave keeps its run 2m + 1 and takes the lower one's
+            const uint32_t p0 = pack_bf16x2(tiles[t][8 * m + 0], tiles[t][8 * m + 1]);
+            const uint32_t p1 = pack_bf16x2(tiles[t][8 * m + 2], tiles[t][8 * m + 3]);
+            const uint32_t q0 = pack_bf16x2(tiles[t][8 * m + 4], tiles[t][8 * m + 5]);
+            const uint32_t q1 = pack_bf16x2(tiles[t][8 * m + 6], tiles[t][8 * m + 7]);
+            const auto s0 = __builtin_amdgcn_permlane32_swap(p0, q0, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(p1, q1, false, false);
+            const uint32_t words[4] = {s0[0], s1[0], s0[1], s1[1]};
+            const int c = 32 * t + 16 * m + 8 * half;
+            if (l32 < valid_rows && c < valid_cols) {
+                if (wide && c + 8 <= valid_cols) {
+                    *reinterpret_cast<uint4 *>(row + c) = make_uint4(words[0], words[1], words[2], words[3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (c + e < valid_cols) {
+                            row[c + e] = static_cast<uint16_t>(words[e >> 1] >> (16 * (e & 1)));
+                        }
+                    }
                 }
             }
         }
     }
-    __builtin_amdgcn_fence(__ATOMIC_ACQ_REL, "wavefront");
-    __builtin_amdgcn_wave_barrier();
 }
 
 template <int TYPE, bool WIDE>
@@ -203,6 +205,12 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         if (lane == 0) {
             lds.item_count = __popcll(mask);
         }
+        if (lane < 4) {
+            lds.produced[lane] = 0;
+        }
+        if (lane < FSC_MULTIPLIERS) {
+            lds.consumed[lane] = 0;
+        }
     }
     if constexpr (TYPE == IQ2_S) {
         expand_iq2s_selectors(lds.codebook, tid, FSC_THREADS);
@@ -223,6 +231,44 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     auto item_field = [&](int item, int field) {
         return __builtin_amdgcn_readfirstlane(reinterpret_cast<const int *>(&lds.items[item])[field]);
     };
+
+    // Stage counters.  Every lane polls the same words (a broadcast read); a wave that has polled FSC_SPIN_LIMIT times
+    // stops waiting, so that a lost count ends in wrong results rather than in a workgroup that never finishes.
+    typedef int i32x4_t __attribute__((ext_vector_type(4)));
+    using SharedCounters = const volatile __attribute__((address_space(3))) i32x4_t *;
+    using SharedCounter = volatile __attribute__((address_space(3))) int *;
+    auto publish = [&](int * counter, int value) __attribute__((always_inline)) {
+        asm volatile("" ::: "memory");   // (the data accesses stay before the count)
+        if (lane == 0) {
+            *(SharedCounter)counter = value;
+        }
+    };
+    auto wait_produced = [&](int need) __attribute__((always_inline)) {
+        for (int polls = 0; polls < FSC_SPIN_LIMIT; ++polls) {
+            const i32x4_t v = *(SharedCounters)&lds.produced[0];
+            if (__builtin_amdgcn_readfirstlane(min(min(v.x, v.y), min(v.z, v.w))) >= need) {
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");   // (the data accesses stay after the count)
+    };
+    auto wait_consumed = [&](int need) __attribute__((always_inline)) {
+        static_assert(FSC_MULTIPLIERS == 8, "two 16-byte reads cover the multipliers' counters");
+        if (need > 0) {
+            for (int polls = 0; polls < FSC_SPIN_LIMIT; ++polls) {
+                const i32x4_t v = *(SharedCounters)&lds.consumed[0];
+                const i32x4_t u = *(SharedCounters)&lds.consumed[4];
+                const int least = min(min(min(v.x, v.y), min(v.z, v.w)), min(min(u.x, u.y), min(u.z, u.w)));
+                if (__builtin_amdgcn_readfirstlane(least) >= need) {
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
+            }
+        }
+        asm volatile("" ::: "memory");
+    };
+    auto next_buffer = [](int buffer) { return buffer + 1 == FSC_BUFFERS ? 0 : buffer + 1; };
 
     if (wave >= FSC_MULTIPLIERS) {
         // ---------------- unpacking wave ----------------
@@ -309,7 +355,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             int exponent = static_cast<int>(__float_as_uint(reach) >> 23);   // biased
             exponent = min(max(exponent, 9), 254);
             if (half == 0) {
-                lds.row_power[c.item & 1][32 * dw + l32] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^S
+                lds.row_power[c.item & 3][32 * dw + l32] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^S
             }
             return __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-S
         };
@@ -376,7 +422,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         };
         float shrink = 1.0f;   // 2^-S of the lane's weight row in the item being unpacked
         // the eight block minima of a Q4_K/Q5_K super-block as the operand of its extra reduction step
-        auto minima_from_header = [&](int parity, const u32x4_t header) {
+        auto minima_from_header = [&](int buffer, const u32x4_t header) {
             int sc, mn[8];
             k45_group_scale_min<0>(header.y, header.z, header.w, sc, mn[0]);
             k45_group_scale_min<1>(header.y, header.z, header.w, sc, mn[1]);
@@ -395,7 +441,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
                                           static_cast<_Float16>(minus * static_cast<float>(mn[2 * i + 1]))};
                     packed[i] = __builtin_bit_cast(uint32_t, pair);
                 }
-                *reinterpret_cast<uint4 *>(&lds.mins[parity][dw * 512 + l32 * 16]) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+                *reinterpret_cast<uint4 *>(&lds.mins[buffer][dw * 512 + l32 * 16]) = make_uint4(packed[0], packed[1], packed[2], packed[3]);
             }
         };
         // stage S (0, 1) of a Q4_K/Q5_K super-block from its fetched inputs -> operand tile `target`
@@ -502,6 +548,8 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         };
         advance(0);
         advance(1);
+        // stage g goes to buffer g % FSC_BUFFERS once the multipliers have read stage g - FSC_BUFFERS
+        int written = 0, buffer = 0;
         StageInputs inputs = {};
         if constexpr (K45) {
             inputs = fetch_inputs(0, 0);
@@ -511,27 +559,29 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         } else {
             unpack(std::integral_constant<int, 0>{}, 0, 0);
         }
+        publish(&lds.produced[dw], ++written);
+        buffer = next_buffer(buffer);
         FSC_LAP(0);
-        __syncthreads();
-        FSC_LAP(1);
         int kb = 0;   // of super-block q within its item
 #pragma unroll 1
         for (int q = 0; q < total; ++q) {
             const int parity = q & 1;
             // (past the last super-block the wave works on a repeat of it: nobody reads what that writes)
-            // while the multipliers work on stage 0 of q: stage 1 of q, then the next super-block's blocks
+            // stage 1 of q
+            wait_consumed(written + 1 - FSC_BUFFERS);
+            FSC_LAP(1);
             if constexpr (K45) {
-                finish_stage(std::integral_constant<int, 1>{}, inputs, 1);
+                finish_stage(std::integral_constant<int, 1>{}, inputs, buffer);
             } else {
-                unpack(std::integral_constant<int, 1>{}, parity, 1);
+                unpack(std::integral_constant<int, 1>{}, parity, buffer);
             }
-            FSC_LAP(2);
+            publish(&lds.produced[dw], ++written);
+            buffer = next_buffer(buffer);
             if constexpr (K45) {
                 inputs = fetch_inputs(0, parity ^ 1);
             }
-            __syncthreads();
-            FSC_LAP(4);
-            // while they work on stage 1: stage 0 of q + 1, which may open the next item
+            FSC_LAP(2);
+            // stage 0 of q + 1, which may open the next item
             if (kb + 1 == super_blocks) {
                 kb = 0;
                 if (q + 1 < total) {
@@ -544,21 +594,23 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             } else {
                 ++kb;
             }
-            FSC_LAP(5);
+            FSC_LAP(3);
+            wait_consumed(written + 1 - FSC_BUFFERS);
+            FSC_LAP(1);
             if constexpr (K45) {
-                minima_from_header(parity ^ 1, inputs.header);
-                finish_stage(std::integral_constant<int, 0>{}, inputs, 0);
+                minima_from_header(buffer, inputs.header);
+                finish_stage(std::integral_constant<int, 0>{}, inputs, buffer);
                 inputs = fetch_inputs(1, parity ^ 1);
             } else {
-                unpack(std::integral_constant<int, 0>{}, parity ^ 1, 0);
+                unpack(std::integral_constant<int, 0>{}, parity ^ 1, buffer);
             }
-            FSC_LAP(6);
+            publish(&lds.produced[dw], ++written);
+            buffer = next_buffer(buffer);
+            FSC_LAP(4);
             // slot `parity` is free (Q4_K/Q5_K: its last inputs are in registers; the others: stage 1 is done):
             // super-block q + 2 goes there
             advance(parity);
-            FSC_LAP(3);
-            __syncthreads();
-            FSC_LAP(4);
+            FSC_LAP(5);
         }
         FSC_LAP_DUMP(1);
         return;
@@ -640,15 +692,16 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         constexpr bool ACTIVE = decltype(active_tag)::value;
 #pragma unroll
         for (int s = 0; s < FSC_STEPS; ++s) {
-            if (s + FSC_W_AHEAD < FSC_STEPS) {
-                read_step(buffer, s + FSC_W_AHEAD, w[(s + FSC_W_AHEAD) % RING]);
+            if constexpr (ACTIVE) {
+                if (s + FSC_W_AHEAD < FSC_STEPS) {
+                    read_step(buffer, s + FSC_W_AHEAD, w[(s + FSC_W_AHEAD) % RING]);
+                }
             }
             const half8_t fragment = rescale(x[s], ratio);
             if constexpr (ACTIVE)
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) {
-                // (weights as the A operand: the lane ends up with one activation row and runs of four neighbouring
-                // columns, which the epilogue stages with 8-byte LDS writes)
+                // (weights as the A operand: the lane ends up with one activation row and runs of four neighbouring columns)
                 acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(w[s % RING][nt], fragment, acc[nt], 0, 0, 0);
             }
             x[s] = load_x(rows_next, next_step + s);
@@ -658,25 +711,21 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         }
     };
     // (a wave without rows in the item keeps requesting activations, which may be the next item's, but leaves the matrix
-    // pipe to the wave it shares the SIMD with)
+    // pipe and the operand tile to the others)
     auto stage = [&](int buffer, int next_step, half2_t ratio, bool active) __attribute__((always_inline)) {
         if (active) {
+#pragma unroll
+            for (int s = 0; s < FSC_W_AHEAD; ++s) {
+                read_step(buffer, s, w[s]);
+            }
             stage_as(std::true_type{}, buffer, next_step, ratio);
         } else {
             stage_as(std::false_type{}, buffer, next_step, ratio);
         }
     };
-    auto read_first_steps = [&](int buffer) {
-#pragma unroll
-        for (int s = 0; s < FSC_W_AHEAD; ++s) {
-            read_step(buffer, s, w[s]);
-        }
-    };
     FSC_LAP(0);
-    __syncthreads();
-    FSC_LAP(1);
-    read_first_steps(0);
     int item = 0, kb = 0;
+    int read = 0, buffer = 0;   // stages read so far; stage g is in buffer g % FSC_BUFFERS
     float ratio_next = load_ratio(rows_next, 0);
 #pragma unroll 1
     for (int q = 0; q < total; ++q) {
@@ -685,43 +734,46 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         if constexpr (K45) {
             sums = load_sums(rows_next, kb);
         }
-        float ratio_f32 = ratio_next;   // (requested a stage ago: needed at once)
-        // a wave without rows in the item multiplies zeros: no branch in the loop, and the matrix pipe draws less
-        // power on zeros, which the clock of the waves that do have rows gains from
+        // 2^E of the lane's row, for the epilogue (requested with every super-block: one that ends an item has it at hand)
+        const float row_power = *reinterpret_cast<const float *>(reinterpret_cast<const uint8_t *>(a.row_power) + rows_next.power_lane);
+        const float ratio_f32 = ratio_next;   // (requested a stage ago: needed at once)
         const bool active = item_field(item, 1) + wave * 32 < item_field(item, 2);
         const half2_t ratio = {static_cast<_Float16>(ratio_f32), static_cast<_Float16>(ratio_f32)};
         // stage 0; requests stage 1 of the same super-block
-        stage(0, kb * 16 + 8, ratio, active);
-        FSC_LAP(2);
-        __syncthreads();
-        FSC_LAP(3);
-        read_first_steps(1);
-        // stage 1; requests stage 0 of the following super-block, which may belong to the next item
-        const bool last_of_item = kb + 1 == super_blocks;
-        const int item_next = last_of_item ? min(item + 1, n_items - 1) : item;
-        const int kb_next = last_of_item ? 0 : kb + 1;
-        rows_next = rows_of(item_next);
-        ratio_next = load_ratio(rows_next, kb_next);
-        stage(1, kb_next * 16, ratio, active);
+        wait_produced(read + 1);
+        FSC_LAP(1);
+        stage(buffer, kb * 16 + 8, ratio, active);
         if constexpr (K45) {
-            // the super-block's extra reduction step: block minima x block sums (slots 8..15 of the instruction are empty)
+            // the super-block's extra reduction step: block minima x block sums (slots 8..15 of the instruction are
+            // empty); the minima lie beside the operand tile of the super-block's first stage
             const half8_t block_sums = rescale(__builtin_bit_cast(half8_t, half != 0 ? make_uint4(0, 0, 0, 0) : sums), ratio);
             if (active)
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) {
-                uint4 minima = *reinterpret_cast<const uint4 *>(&lds.mins[q & 1][nt * 512 + l32 * 16]);
+                uint4 minima = *reinterpret_cast<const uint4 *>(&lds.mins[buffer][nt * 512 + l32 * 16]);
                 if (half != 0) {
                     minima = make_uint4(0, 0, 0, 0);
                 }
                 acc[nt] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, minima), block_sums, acc[nt], 0, 0, 0);
             }
         }
-        FSC_LAP(4);
-        __syncthreads();
+        publish(&lds.consumed[wave], ++read);
+        buffer = next_buffer(buffer);
+        FSC_LAP(2);
+        // stage 1; requests stage 0 of the following super-block, which may belong to the next item
+        const bool last_of_item = kb + 1 == super_blocks;
+        const int item_next = last_of_item ? min(item + 1, n_items - 1) : item;
+        const int kb_next = last_of_item ? 0 : kb + 1;
+        rows_next = rows_of(item_next);
+        ratio_next = load_ratio(rows_next, kb_next);
+        wait_produced(read + 1);
+        FSC_LAP(1);
+        stage(buffer, kb_next * 16, ratio, active);
+        publish(&lds.consumed[wave], ++read);
+        buffer = next_buffer(buffer);
         FSC_LAP(3);
         if (last_of_item) {
-            // The item is complete: scale by 2^(E[r] + S[n]) and store, 32 rows x 64 columns at a time through this
-            // wave's staging area, while the unpacking waves work on the next item.
+            // The item is complete: scale by 2^(E[r] + S[n]) and store, while the unpacking waves work on the next item.
             const int row_start = item_field(item, 1);
             const int row_end = item_field(item, 2);
             const int tile = item_field(item, 3);
@@ -734,36 +786,29 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             asm volatile("" : "+v"(lane_here));
             const int l32_here = lane_here & 31, half_here = lane_here >> 5;
             if (r0 < row_end) {
-                const float row_power = a.row_power[min(r0 + l32_here, a.rows_padded - 1)];
 #pragma unroll
-                for (int pair = 0; pair < 2; ++pair) {
+                for (int nt = 0; nt < FWD_NT; ++nt) {
 #pragma unroll
-                    for (int t = 0; t < 2; ++t) {
-                        const int nt = 2 * pair + t;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) {
-                            const float4 column_power =
-                                *reinterpret_cast<const float4 *>(&lds.row_power[item & 1][nt * 32 + 8 * j + 4 * half_here]);
-                            acc[nt][4 * j + 0] *= row_power * column_power.x;
-                            acc[nt][4 * j + 1] *= row_power * column_power.y;
-                            acc[nt][4 * j + 2] *= row_power * column_power.z;
-                            acc[nt][4 * j + 3] *= row_power * column_power.w;
-                        }
+                    for (int j = 0; j < 4; ++j) {
+                        const float4 column_power =
+                            *reinterpret_cast<const float4 *>(&lds.row_power[item & 3][nt * 32 + 8 * j + 4 * half_here]);
+                        acc[nt][4 * j + 0] *= row_power * column_power.x;
+                        acc[nt][4 * j + 1] *= row_power * column_power.y;
+                        acc[nt][4 * j + 2] *= row_power * column_power.z;
+                        acc[nt][4 * j + 3] *= row_power * column_power.w;
                     }
-                    const v16f (&tiles)[2] = *reinterpret_cast<const v16f (*)[2]>(&acc[2 * pair]);
-                    store_rows_32x64(lds.staging[wave], tiles, y + static_cast<int64_t>(r0) * a.out_features + n0 + 64 * pair,
-                                     a.out_features, row_end - r0, a.out_features - n0 - 64 * pair, lane_here);
                 }
+                store_rows_32x128(acc, y + static_cast<int64_t>(r0) * a.out_features + n0, a.out_features, row_end - r0,
+                                  a.out_features - n0, lane_here);
             }
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) acc[nt] = zero;
             ++item;
             kb = 0;
-            FSC_LAP(5);
+            FSC_LAP(4);
         } else {
             ++kb;
         }
-        read_first_steps(0);   // of the next super-block (a stale tile after the last one: never used)
     }
     FSC_LAP_DUMP(0);
 }

@@ -15,10 +15,13 @@ namespace tgo {
 //                   weight, each normalised by a power of two per row and rounded to fp16 once.  The matrix
 //                   instruction then accumulates the whole reduction and no vector instruction touches a result
 //                   before the epilogue (tgo_forward_scaled.hip): the only kind whose bound is the matrix pipe.
-//   OPERAND_AUTO    (default) the fastest kind measured per format.
+//   OPERAND_AUTO    (default) scaled operands for calls with enough tasks to fill the chip with its 256-row x
+//                   128-column tiles, otherwise exact fp16 for IQ2_S and int8 for the other formats (their smaller
+//                   tiles spread a small call over more CUs).
 // `quant_type` 0 stands for a workspace that is quantized without knowing the format it will be used with
-// (tgo_quantize_q8_1 without a format): int8 unless another kind is forced.  The activation workspace is written for
-// one kind of operand and records which (Q8Workspace::tag); it must be consumed as that kind.
+// (tgo_quantize_q8_1, tgo_mmq_forward_prepared): int8 unless exact fp16 is forced.  The activation workspace is
+// written for one kind of operand and records which (Q8Workspace::tag); it must be consumed as that kind.  A call
+// reads the setting once, so a change by another thread never splits a call between two kinds.
 enum ForwardOperand : int { OPERAND_INT8 = 0, OPERAND_HALF = 1, OPERAND_AUTO = 2, OPERAND_SCALED = 3 };
 int forward_operand_setting();
 void set_forward_operand_setting(int operand);
@@ -26,14 +29,21 @@ void set_forward_operand_setting(int operand);
 static constexpr bool scaled_forward_format(int quant_type) {
     return quant_type == 11 || quant_type == 12 || quant_type == 13 || quant_type == 14 || quant_type == 22;
 }
-// The operand kind a call of this format uses under the current setting (never OPERAND_AUTO).
-static inline int forward_operand_kind(int quant_type) {
+// Fewest (256-row x 128-column) tiles for which OPERAND_AUTO picks the scaled kernel: one workgroup per CU runs them,
+// so half a chip's worth is where it starts to beat the kernels with smaller tiles (dense 512 x 4096: 64 tiles, a
+// tie; 4096 x 2048: 256 tiles, 12 % faster).
+constexpr int64_t SCALED_AUTO_MIN_TILES = 128;
+// The operand kind a call of this format and size uses under the current setting (never OPERAND_AUTO).  Grouped
+// calls pass their total rows: the tiles of a ragged list are at least that many.
+static inline int forward_operand_kind(int quant_type, int64_t rows = 0, int64_t out_features = 0, int projections = 1) {
     const int setting = forward_operand_setting();
+    const int exact = quant_type == 22 ? OPERAND_HALF : OPERAND_INT8;
     if (setting == OPERAND_SCALED) {
-        return scaled_forward_format(quant_type) ? OPERAND_SCALED : quant_type == 22 ? OPERAND_HALF : OPERAND_INT8;
+        return scaled_forward_format(quant_type) ? OPERAND_SCALED : exact;
     }
     if (setting == OPERAND_AUTO) {
-        return quant_type == 22 ? OPERAND_HALF : OPERAND_INT8;
+        const int64_t tiles = ((rows + 255) / 256) * ((out_features + 127) / 128) * projections;
+        return scaled_forward_format(quant_type) && tiles >= SCALED_AUTO_MIN_TILES ? OPERAND_SCALED : exact;
     }
     return setting;
 }
@@ -42,7 +52,7 @@ static inline int forward_operand_kind(int quant_type) {
 static constexpr int half_forward_waves(int quant_type) { return quant_type == 14 || quant_type == 22 ? 8 : 4; }
 // Row tile of one forward task; the task list is built for these.  int8 operands: 256 rows for the formats whose
 // weights unpack into two int8 planes (Q6_K = 14, IQ2_S = 22), 128 rows for the single-plane ones; exact fp16
-// operands: 32 rows per wave of the format's workgroup; scaled operands: 256 (four multiplying waves of 64 rows).
+// operands: 32 rows per wave of the format's workgroup; scaled operands: 256 (eight multiplying waves of 32 rows).
 static constexpr int forward_row_tile(int quant_type, int operand_kind) {
     return operand_kind == OPERAND_SCALED ? 256
            : operand_kind == OPERAND_HALF ? 32 * half_forward_waves(quant_type)
@@ -215,6 +225,8 @@ hipError_t launch_dequant_bf16(const uint8_t * packed, uint16_t * out, int64_t r
 hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, int64_t rows,
                                 int64_t in_features, hipStream_t stream, const int64_t * gather = nullptr,
                                 int64_t input_rows = 0, const TaskBuild * build = nullptr);
+// Turns `count` bf16 outputs into NaN when the workspace's tag is not the layout of `ws` (runs behind the multiply kernel).
+hipError_t launch_workspace_guard(const Q8Workspace & ws, uint16_t * out, int64_t count, hipStream_t stream);
 hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float * sum, int64_t rows,
                             int64_t in_features, hipStream_t stream);
 

@@ -52,6 +52,7 @@ lib.tgo_profile_enable.argtypes = [_int]
 lib.tgo_profile_read.argtypes = [_int, ctypes.POINTER(ctypes.c_double), ctypes.POINTER(ctypes.c_int64)]
 lib.tgo_set_forward_operand.argtypes = [_int]
 lib.tgo_forward_operand.argtypes = []
+lib.tgo_forward_operand_for.argtypes = [_int, _i64, _i64, _int]
 
 KERNEL_IDS = {
     "quantize": 0, "build_tasks": 1, "forward": 2, "grad_input": 3, "dequant": 4, "forward_gemv": 5,
@@ -84,6 +85,7 @@ EXPORTS = (
     "tgo_profile_read",
     "tgo_set_forward_operand",
     "tgo_forward_operand",
+    "tgo_forward_operand_for",
 )
 
 OPERANDS = {"int8": 0, "half": 1, "auto": 2, "scaled": 3}
@@ -91,14 +93,19 @@ OPERANDS = {"int8": 0, "half": 1, "auto": 2, "scaled": 3}
 
 def set_forward_operand(operand: str) -> None:
     """Matrix operands of the MFMA forward kernels: "int8", "half" (fp16 numbers holding the exact integers),
-    "scaled" (exact integer weights x the dequantized q8_1 activations as fp16, scaled once per super-block: the
-    kind bounded by the matrix pipe; Q6_K has no such kernel and keeps int8), or "auto" (the default: the
-    fastest kind measured per format)."""
+    "scaled" (dequantized activations and weights as fp16, normalised per row: the kind bounded by the matrix
+    pipe), or "auto" (the default: scaled for calls that fill the chip, otherwise half for IQ2_S and int8 for
+    the other formats)."""
     check(lib.tgo_set_forward_operand(OPERANDS[operand]))
 
 
 def forward_operand() -> str:
     return {value: name for name, value in OPERANDS.items()}[lib.tgo_forward_operand()]
+
+
+def forward_operand_for(quant_type: int, rows: int, out_features: int, projections: int = 1) -> str:
+    """The kind a forward call of this format and shape uses under the current setting (never "auto")."""
+    return {value: name for name, value in OPERANDS.items()}[lib.tgo_forward_operand_for(quant_type, rows, out_features, projections)]
 
 
 def profile_read(kernel: str) -> tuple[float, int]:

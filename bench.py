@@ -110,8 +110,7 @@ def measure_pair_format(device, name, qtype, steps=10, warmup=3):
     record = {
         "workload": f"grouped_mmq_pair fwd+bwd, gate+up {name} [512,2048], same routing as the headline workload",
         "value": flops / (elapsed / steps) / 1e12, "unit": "TFLOP/s", "ms_per_step": elapsed / steps * 1e3, "steps": steps,
-        "forward_operands": "fp16 numbers holding the exact integers" if _native.forward_operand() == "half" or
-        (_native.forward_operand() == "auto" and qtype == 22) else "int8",
+        "forward_operands": _native.forward_operand_for(qtype, w["rows"], w["n"], 2),
         "kernels_us": {k: total / launches * 1e3 for k, (total, launches) in kernels.items() if launches},
     }
     del w
@@ -684,14 +683,22 @@ def main() -> None:
     active = w["indices"].numel()
     weight_bytes = 2 * active * n * (k // 256) * _native.lib.tgo_block_bytes(w["qtype"])
 
-    # the forward multiplies int8 operands, or fp16 numbers holding the same integers (the library's choice for IQ2_S)
-    half_operands = args.operand in ("half", "scaled") or (args.operand == "auto" and args.quant == "IQ2_S")
+    # the forward multiplies int8 operands, fp16 numbers holding the same integers, or fp16 numbers that carry the
+    # scales as well: the library's choice for this call unless --operand forces one
+    operand_kind = _native.forward_operand_for(w["qtype"], rows, n, 2)
+    half_operands = operand_kind in ("half", "scaled")
     forward_peak = PEAK["bf16"] if half_operands else PEAK["int8"]   # fp16 and bf16 share the dense matrix peak
+    forward_dtype = {"int8": "int8", "half": "fp16 holding exact integers", "scaled": "fp16 carrying the scales"}[operand_kind]
+    # bytes the quantizer moves: bf16 in; int8 or fp16 values, an fp32 scale and sum per 32 values, and for the scaled
+    # operands a power of two and eight fp16 block sums per 256 values and a power of two per row out
+    quantize_bytes = rows * k * 2 + rows * k * (2 if half_operands else 1) + 2 * rows * (k // 32) * 4
+    if operand_kind == "scaled":
+        quantize_bytes += rows * (k // 256) * 20 + rows * 4
     # per-launch algorithmic work of each profiled kernel
     per_launch = {
         "forward": ("mfma", 2 * flops_projection / 1e12, forward_peak, "TFLOP/s"),  # both projections per launch
         "grad_input": ("mfma", 2 * flops_projection / 1e12, PEAK["bf16"], "TFLOP/s"),  # both products per launch
-        "quantize": ("hbm", (rows * k * 2 + rows * k + 2 * rows * (k // 32) * 4) / 1e9, PEAK["hbm"], "GB/s"),
+        "quantize": ("hbm", quantize_bytes / 1e9, PEAK["hbm"], "GB/s"),
         "pack_cotangent": ("hbm", 2 * 2 * rows * n * 2 / 1e9, PEAK["hbm"], "GB/s"),  # both cotangents read + written
     }
     breakdown = {}
@@ -735,7 +742,7 @@ def main() -> None:
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": ("fp16 holding exact integers" if half_operands else "int8") + " (forward dot products) / bf16 (grad-input), fp32 accumulate",
+        "dtype": forward_dtype + " (forward dot products) / bf16 (grad-input), fp32 accumulate",
         "data": "synthetic",
         "config": {
             "workload": f"grouped_mmq_pair fwd+bwd: 256 experts, gate+up {args.quant} [512,2048], T=8192 x top-8 "
@@ -743,6 +750,7 @@ def main() -> None:
             "rows": rows,
             "active_experts": active,
             "quant_type": args.quant,
+            "forward_operands": operand_kind,
         },
         "weight_GBps": weight_bytes * 2 / (elapsed / args.steps) / 1e9,  # read once forward, once backward
         "roofline": roofline,

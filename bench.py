@@ -23,7 +23,7 @@ import time
 from pathlib import Path
 
 ROOT = Path(__file__).resolve().parent
-for entry in (ROOT, ROOT / "torch-ggml-ops_amd"):
+for entry in (ROOT, ROOT / "torch-ggml-ops_amd", ROOT / "tests"):   # (tests/: the synthetic blocks and routing)
     if str(entry) not in sys.path:
         sys.path.insert(0, str(entry))
 
@@ -38,7 +38,7 @@ VALU_BOUND_INT8 = PEAK["fp32_vector"] / 4 / 2 * 64  # TOP/s: 1258.4, i.e. 25.2 %
 
 
 def build_pair_workload(device, tokens=8192, experts=256, top_k=8, n=512, k=2048, qtype=13, seed=2024):
-    from torch_ggml_ops import synth
+    import synth
 
     token_of_row, indices, offsets, _ = synth.zipf_routing(tokens, experts, top_k, seed, device=device)
     generator = torch.Generator(device=device).manual_seed(seed + 1)
@@ -161,7 +161,8 @@ def measure_decode(args, device) -> dict:
     Every call uses a different seeded routing out of eight, so successive calls touch different experts
     and the weights (392 MB in total) do not stay in the 256 MB last-level cache."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import _native, synth
+    import synth
+    from torch_ggml_ops import _native
 
     experts, top_k = 256, 8
     gate = synth.random_packed_weight(synth.IQ2_S, (experts, 512), 2048, 11, device=device)
@@ -299,7 +300,7 @@ def run_multi(args, device) -> None:
     """Several dense projections of one input (attention q/k/v of a GQA layer: 4096 -> 4096, 1024, 1024, Q4_K,
     4096 token rows): three `mmq` calls against one `mmq_multi`, which quantizes the activations once."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import synth
+    import synth
 
     rows, k, widths = 4096, 4096, (4096, 1024, 1024)
     generator = torch.Generator(device=device).manual_seed(9)
@@ -350,7 +351,8 @@ def run_dense(args, device) -> None:
     K = 2048, forward and grad-input; kernel time per call (quantize + multiply, pack + multiply) and TFLOP/s or,
     for the bandwidth-bound small-M rows, weight GB/s."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import synth, _native
+    import synth
+    from torch_ggml_ops import _native
 
     k = 2048
     names = {11: "Q3_K", 12: "Q4_K", 13: "Q5_K", 14: "Q6_K", 22: "IQ2_S"}
@@ -400,7 +402,8 @@ def measure_down(args, device) -> dict:
     """The down projection of the default workload's model: grouped_mmq, 256 experts, Q4_K [2048, 512],
     4096 tokens x top-8 with the same skewed routing (32 768 rows); forward and grad-input kernel times."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import synth, _native
+    import synth
+    from torch_ggml_ops import _native
 
     experts, n, k, qtype = 256, 2048, 512, 12
     token_of_row, indices, offsets, _ = synth.zipf_routing(4096, experts, 8, 11, device=device)
@@ -466,7 +469,7 @@ def run_gathered(args, device) -> None:
     """The default workload's forward from unsorted token activations: `index_select` to expert-sorted rows
     followed by `grouped_mmq_pair`, against `grouped_mmq_pair_gathered`, whose quantizer reads the token rows."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import synth
+    import synth
 
     tokens, experts, top_k, n, k, qtype, seed = 8192, 256, 8, 512, 2048, 13, 2024
     token_of_row, indices, offsets, _ = synth.zipf_routing(tokens, experts, top_k, seed, device=device)
@@ -509,7 +512,8 @@ def run_layer(args, device) -> None:
     """Forward of one SwiGLU mixture-of-experts layer from token activations to token outputs (`moe_layer`):
     routing sort, gathered gate+up pair, activation, down projection, routing-weighted combine."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import _native, synth
+    import synth
+    from torch_ggml_ops import _native
 
     tokens, experts, top_k, intermediate, features, qtype, seed = 8192, 256, 8, 512, 2048, 13, 2024
     token_of_row, indices, offsets, _ = synth.zipf_routing(tokens, experts, top_k, seed, device=device)

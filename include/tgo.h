@@ -206,7 +206,8 @@ int tgo_grouped_mmq_grad_input(const void * grad_output_first, const void * grad
  *   bf16( row_weight[r] * grad_tokens[row_token[r], :] )        (fp32 product, one rounding)
  * with grad_tokens bf16 [tokens, out_features] the gradient of the layer's per-token output, row_token int64
  * [rows] the token of each expert-sorted row and row_weight fp32 [rows] its routing weight; a row whose token
- * lies outside [0, tokens) has a zero cotangent.  The expert-sorted cotangent that the caller would otherwise
+ * lies outside [0, tokens) has a zero cotangent.  (One token and weight per row: this is the backward of
+ * tgo_moe_combine only for slot_rows that name every row at most once.)  The expert-sorted cotangent that the caller would otherwise
  * build from the gradient of tgo_moe_combine (rows x out_features bf16, written and read again) is never
  * materialised.  Same workspace as tgo_grouped_mmq_grad_input with one source.  No counterpart in the reference,
  * which leaves the combine and its gradient to the caller (torch_ggml_ops/grouped_mmq.py:216). */

@@ -18,7 +18,8 @@ ROOT = Path(__file__).resolve().parents[1]
 @pytest.fixture(scope="module")
 def package():
     import torch_ggml_ops
-    from torch_ggml_ops import _native, _validate, synth
+    import synth
+    from torch_ggml_ops import _native, _validate
 
     return torch_ggml_ops, _native, _validate, synth
 

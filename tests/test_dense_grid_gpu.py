@@ -29,7 +29,7 @@ EDGE_ROWS = (0, 1, 31, 32, 33, 63, 64, 127, 128, 129, 255, 256, 257, 511, 512, 2
 @pytest.fixture(scope="module")
 def ops():
     import torch_ggml_ops
-    from torch_ggml_ops import synth
+    import synth
 
     assert torch.cuda.is_available()
     return torch_ggml_ops, synth

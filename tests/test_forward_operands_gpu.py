@@ -22,7 +22,8 @@ FORWARD_TOLERANCE = 1e-2   # against dequantize-then-matmul, as in the dense tes
 @pytest.fixture(scope="module")
 def ops():
     import torch_ggml_ops
-    from torch_ggml_ops import _native, synth
+    import synth
+    from torch_ggml_ops import _native
 
     assert torch.cuda.is_available()
     return torch_ggml_ops, _native, synth

@@ -23,7 +23,7 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def ops():
     import torch_ggml_ops
-    from torch_ggml_ops import synth
+    import synth
 
     assert torch.cuda.is_available()
     return torch_ggml_ops, synth

@@ -171,7 +171,7 @@ def test_file_to_device_to_grouped_operator(tmp_path):
     """Experts written to a GGUF file, read back and uploaded in chunks, give the same operator output bit for
     bit as the same bytes uploaded directly."""
     import torch_ggml_ops as tgo
-    from torch_ggml_ops import synth
+    import synth
 
     experts, n, k, qtype = 4, 96, 512, 13
     host = synth.random_packed_weight(qtype, (experts, n), k, seed=77)

@@ -20,7 +20,7 @@ BOUNDARY_SIZES = (1, 15, 16, 17, 63, 64, 65, 127, 128, 129)
 @pytest.fixture(scope="module")
 def ops():
     import torch_ggml_ops
-    from torch_ggml_ops import synth
+    import synth
 
     assert torch.cuda.is_available()
     return torch_ggml_ops, synth

@@ -204,7 +204,7 @@ def test_single_value_accessor_agrees_with_row_decoder(oracle):
 
 
 def _random_rows(rng, qtype, rows, in_features, subnormal_scales=False):
-    from torch_ggml_ops import synth
+    import synth
 
     block = synth.BLOCK_BYTES[qtype]
     count = rows * (in_features // 256)
@@ -312,7 +312,7 @@ def _zeroed_quants(qtype, packed):
 
 @pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_mmq_forward_equals_dequantized_operands_matmul(oracle, qtype):
-    from torch_ggml_ops import synth
+    import synth
 
     rng = np.random.default_rng(200 + qtype)
     rows, n, k = 5, 7, 512
@@ -381,7 +381,7 @@ def test_half_scale_mode_equals_numpy_restatement_and_stays_close_to_fp32_mode(o
     float64 evaluation with float16 casts in those four places, and its distance from the fp32-scale algebra (what the
     library computes) is measured: a relative error of at most 2^-11 per factor, far inside the 1e-2 the operator
     promises."""
-    from torch_ggml_ops import synth
+    import synth
     from helpers import max_rel_to_peak, nrmse
 
     rng = np.random.default_rng(900 + qtype)
@@ -411,7 +411,7 @@ def test_half_scale_mode_equals_numpy_restatement_and_stays_close_to_fp32_mode(o
 
 @pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_linear_and_grad_input_equal_float64_matmul(oracle, qtype):
-    from torch_ggml_ops import synth
+    import synth
 
     rng = np.random.default_rng(300 + qtype)
     rows, n, k = 4, 9, 256
@@ -429,7 +429,7 @@ def test_linear_and_grad_input_equal_float64_matmul(oracle, qtype):
 
 @pytest.mark.parametrize("qtype", ALL_TYPES)
 def test_one_hot_cotangent_reproduces_weight_row(oracle, qtype):
-    from torch_ggml_ops import synth
+    import synth
 
     packed = synth.random_packed_weight(qtype, (5,), 512, seed=80 + qtype).numpy()
     dy = np.zeros((1, 5), dtype=np.float32)
@@ -443,10 +443,26 @@ def test_one_hot_cotangent_reproduces_weight_row(oracle, qtype):
 
 
 def test_grouped_helper_skips_invalid_groups(oracle):
-    from torch_ggml_ops import synth
+    import synth
 
     packed = synth.random_packed_weight(Q4_K, (3, 4), 256, seed=1).numpy()
     x = _bf16_bits(np.ones((6, 256), dtype=np.float32))
     out = oracle.grouped(oracle.linear_forward, Q4_K, x, packed, [0, 7, 2], [2, 4, 6], 4, 256, 4)
     assert np.isfinite(out[0:2]).all() and np.isnan(out[2:4]).all() and np.isfinite(out[4:6]).all()
     np.testing.assert_array_equal(out[4:6], oracle.linear_forward(Q4_K, x[4:6], packed[2], 4, 256))
+
+
+def test_round_half_up_equals_roundf_on_every_product_the_quantizer_can_form():
+    """The GPU quantizer rounds |x * (127 / amax)| with the hardware's round-half-up conversion, the reference with
+    roundf (csrc/mmq_core.cuh:186).  On non-negative inputs the two differ at one float only, the largest one below
+    0.5 (0x3EFFFFFF), if the conversion adds 0.5 in fp32.  x and amax are bf16 values and powers of two cancel in the
+    product, so all products are covered by amax in [1, 2) and x <= amax: none of them is that float."""
+    target = np.array([0x3EFFFFFF], dtype=np.uint32).view(np.float32)[0]
+    mantissas = (1.0 + np.arange(128, dtype=np.float64) / 128.0)
+    amax = mantissas.astype(np.float32)                                   # [128]
+    d_inv = (np.float32(127.0) / amax).astype(np.float32)
+    exponents = 2.0 ** np.arange(-140, 1, dtype=np.float64)
+    x = (mantissas[None, :] * exponents[:, None]).astype(np.float32).reshape(-1)   # every bf16 magnitude below 2
+    product = (x[None, :] * d_inv[:, None]).astype(np.float32)
+    reachable = x[None, :] <= amax[:, None]
+    assert not np.any(reachable & (product == target))

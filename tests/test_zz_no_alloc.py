@@ -17,7 +17,8 @@ pytestmark = pytest.mark.gpu
 @pytest.fixture(scope="module")
 def native():
     import torch_ggml_ops  # noqa: F401
-    from torch_ggml_ops import _native, synth
+    import synth
+    from torch_ggml_ops import _native
 
     assert torch.cuda.is_available()
     return _native, synth

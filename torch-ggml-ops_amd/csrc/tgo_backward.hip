@@ -223,13 +223,7 @@ TGO_DEVICE void task_segment(const BackwardArgs & a, int & first, int & tasks) {
 // requested as aligned 16-byte units while the previous step multiplies, like those of Q4_K / Q5_K, instead of
 // being copied two bytes at a time between the multiplications and the decoding.
 template <int TYPE, bool SHORT, bool WIDE>
-#ifndef TGO_SHORT_OCC
-#define TGO_SHORT_OCC 3
-#endif
-#ifndef TGO_SHORT_DEPTH
-#define TGO_SHORT_DEPTH 1
-#endif
-__global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_grad_input_kernel(const BackwardArgs a) {
+__global__ __launch_bounds__(BWD_THREADS, SHORT ? 3 : 2) void mmq_grad_input_kernel(const BackwardArgs a) {
     using F = Format<TYPE>;
     constexpr int KT = SHORT ? 1 : 4;   // 32-column tiles per wave
     constexpr bool FAST_K45 = TYPE == Q4_K || TYPE == Q5_K;
@@ -428,11 +422,11 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
         __syncthreads();   // tile visible
     };
 
-    if constexpr (SHORT && FAST_K45 && TGO_SHORT_DEPTH > 0) {
+    if constexpr (SHORT && FAST_K45) {
         // The multiplications of a step are too short here to cover a memory round trip, so the packed blocks travel
         // DEPTH steps ahead through a ring of register sets and the cotangent fragments two steps ahead; steps past
         // the end repeat the last one (harmless re-reads instead of branches around loads).
-        constexpr int DEPTH = TGO_SHORT_DEPTH > 0 ? TGO_SHORT_DEPTH : 1;
+        constexpr int DEPTH = 1;
         const int last = step_end - 1;
         u32x4 ring[DEPTH][RAW_REGS];
         u32x4 cot[2][2][4] = {};
@@ -626,9 +620,8 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
         __syncthreads();
         auto run = [&](auto active_tag) __attribute__((always_inline)) {
             constexpr bool ACTIVE = decltype(active_tag)::value;
-#ifndef TGO_IL_VALU
-#define TGO_IL_VALU 12
-#endif
+            // vector instructions scheduled behind each matrix instruction of a step (12: measured best of 0..16)
+            constexpr int INTERLEAVED_VALU = 12;
 #pragma unroll 1
             for (int step = step_begin; step < last; ++step) {
                 const int parity = (step - step_begin) & 1;
@@ -656,12 +649,12 @@ __global__ __launch_bounds__(BWD_THREADS, SHORT ? TGO_SHORT_OCC : 2) void mmq_gr
                     if (s == 3) {
                         request(step + 3);
                     }
-                    if constexpr (ACTIVE && !SHORT && TGO_IL_VALU > 0) {
+                    if constexpr (ACTIVE && !SHORT) {
                         // one matrix instruction, then a run of the vector instructions that share its chunk
 #pragma unroll
                         for (int i = 0; i < 2 * KT; ++i) {
                             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                            __builtin_amdgcn_sched_group_barrier(0x002, TGO_IL_VALU, 0);
+                            __builtin_amdgcn_sched_group_barrier(0x002, INTERLEAVED_VALU, 0);
                         }
                     }
                 }

@@ -239,6 +239,10 @@ def grouped_mmq_combine(
     is gathered and scaled by the routing weight while the projection's cotangent is packed, so the
     expert-sorted gradient of the separate calls (``rows x out_features`` bf16 written, then read) never exists;
     the result equals theirs bit for bit.  Also differentiable with respect to ``slot_weights``.
+
+    Every expert-sorted row may be named by at most one (token, choice) slot of ``slot_rows``, as ``route``
+    guarantees: the backward inverts ``slot_rows`` into one (token, weight) per row, so a row named twice would keep
+    one of its slots only, whereas the forward (and the separate ``moe_combine``) adds both.
     """
     output, _rows = torch.ops.torch_ggml_ops.grouped_mmq_combine.default(
         input, packed_weight, expert_indices, expert_offsets, slot_rows, slot_weights, int(quant_type), int(out_features)

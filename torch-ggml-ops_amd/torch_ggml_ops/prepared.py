@@ -3,7 +3,13 @@
 ``mmq`` quantizes its input to q8_1 blocks on every call.  When the same activations feed
 several packed weights (q/k/v, a shared expert's gate/up), that work and its HBM traffic can be
 paid once: ``quantize_q8_1`` returns the library's q8_1 workspace as an opaque uint8 tensor and
-``mmq_prepared`` runs only the matmul half on it.  Results are bit-identical to ``mmq``.
+``mmq_prepared`` runs only the matmul half on it.  A workspace that is quantized before its format is
+known holds int8 operands (exact fp16 ones when ``set_forward_operand("half")`` forces them), so the
+results are bit-identical to ``mmq`` wherever ``mmq`` multiplies the same kind: formats other than IQ2_S
+in calls below the size at which ``mmq`` switches to its scaled operands (``forward_operand_for``).
+Otherwise they are the same q8_1 algebra with another summation order or operand rounding (IQ2_S: exact
+fp16 in ``mmq``, int8 here, whose kernel is about a third slower for that format; large calls: scaled
+operands in ``mmq``, up to 8e-4 of the largest output apart).
 
 The reference has no such operator; it lists this reuse as its next optimisation
 (docs/mmq_fwd_optimization.md:299-307).  ``mmq_multi`` is the convenience wrapper with autograd
@@ -49,10 +55,12 @@ def _quantize_device(input: torch.Tensor) -> torch.Tensor:
 
 @torch.library.register_fake("torch_ggml_ops::quantize_q8_1")
 def _quantize_fake(input):
+    # (tgo_q8_workspace_bytes: two bytes per value, two fp32 per 32 values, 20 bytes per 256 values, 4 per row, 1 KiB)
     in_features = input.shape[-1]
     rows = input.numel() // in_features
     padded = (rows + 31) // 32 * 32
-    return input.new_empty((padded * in_features + 8 * padded * (in_features // 32) + 1024,), dtype=torch.uint8)
+    size = 2 * padded * in_features + 8 * padded * (in_features // 32) + 20 * padded * (in_features // 256) + 4 * padded + 1024
+    return input.new_empty((size,), dtype=torch.uint8)
 
 
 @torch.library.impl("torch_ggml_ops::mmq_prepared", "CUDA")

@@ -589,7 +589,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     if (ws.rows_padded >= (1 << 24) || in_features >= (1 << 24)) {
         return hipErrorInvalidValue;   // lane offsets are formed with 24-bit multiplies
     }
-    ForwardArgs args;
+    ForwardArgs args = {};
     args.packed = packed;
     args.packed_second = packed_second;
     args.y_second = output_second;

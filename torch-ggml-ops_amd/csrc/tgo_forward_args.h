@@ -39,6 +39,7 @@ struct ForwardArgs {
     int task_slots;
     int dense_row_tile;   // dense calls: rows per workgroup (the format's row tile, or 32 when that fills the chip better)
     int wide;             // 2-byte aligned formats: the weights may be fetched as aligned 16-byte units (wide_stage_ok)
+    int early_only;       // grouped calls: 1 = this launch runs the tasks listed before the short ones, another kernel the rest
 };
 
 // The (column tile, projection, task) of this workgroup; false when the slot holds no task.
@@ -46,9 +47,11 @@ struct ForwardArgs {
 TGO_DEVICE bool forward_pick_linear(const ForwardArgs & a, int linear, int & n_tile, bool & second, int & expert,
                                     int & row_start, int & row_end) {
     int task;
-    const int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + a.dense_row_tile - 1) / a.dense_row_tile;
+    int tasks = a.task_count != nullptr ? a.task_count[0] : (a.rows + a.dense_row_tile - 1) / a.dense_row_tile;
     if (a.task_count != nullptr) {
-        xcd_chunk(linear, a.n_tiles * a.projections, tasks, min(a.task_early[0], tasks), n_tile, task);
+        const int early = min(a.task_early[0], tasks);
+        tasks = a.early_only != 0 ? early : tasks;
+        xcd_chunk(linear, a.n_tiles * a.projections, tasks, early, n_tile, task);
     } else {
         xcd_tile<FWD_XCD_RUN>(linear, a.n_tiles * a.projections, tasks, n_tile, task);
     }

@@ -67,6 +67,16 @@ def measured_traffic(kernel):
         return None
 
 
+def measured_pipe_busy(kernel):
+    """Fraction of the kernel's time its matrix and vector pipes were busy on the default workload, from the committed
+    counter summary (rocprofv3 SQ_VALU_MFMA_BUSY_CYCLES, SQ_ACTIVE_INST_VALU and SQ_BUSY_CYCLES); None if absent."""
+    path = ROOT / "profiles" / "grouped_pair_q5k_pipe_utilisation.json"
+    try:
+        return json.loads(path.read_text())["kernels"][kernel]
+    except (OSError, KeyError, ValueError):
+        return None
+
+
 def decode_traffic():
     """HBM bytes per launch of the single-row kernel on the 132 MB dense matrix (the decode workload's best case):
     FETCH_SIZE from the committed counter summary plus the bf16 output row; None if absent."""
@@ -269,15 +279,48 @@ def measure_decode(args, device) -> dict:
         kernel_ms, launches = _native.profile_read("forward_gemv")
         _native.lib.tgo_profile_enable(0)
         report[f"dense_Q4_K_{big_n}x{big_k}_M{m}"] = {
+            "name": f"{big_n}x{big_k}_M{m}",
             "weight_MB": big_bytes / 1e6,
             "us_per_call": elapsed / args.steps * 1e6,
             "gemv_kernel_us": kernel_ms / launches * 1e3,
             "GBps_gemv_kernel": big_bytes / (kernel_ms / launches * 1e-3) / 1e9,
         }
+    if "skewed" in cases:
+        # a small batch that the host cannot tell from an even one: every expert listed, one group of 200 rows and 56
+        # single rows (the kernel family is chosen from rows and listed groups; the large group's eight-row tasks share
+        # the expert's weights through the L2)
+        sizes = [0] * experts
+        sizes[7] = 200
+        for i in range(56):
+            sizes[20 + 3 * i] = 1
+        offsets = torch.tensor(sizes, dtype=torch.int64).cumsum(0).to(torch.int32).to(device)
+        indices = torch.arange(experts, dtype=torch.int64, device=device)
+        x = torch.randn(sum(sizes), 2048, device=device, generator=generator).to(torch.bfloat16)
+        for _ in range(args.warmup):
+            tgo.grouped_mmq_pair(x, gate, up, indices, offsets, synth.IQ2_S, 512)
+        torch.cuda.synchronize()
+        _native.lib.tgo_profile_enable(1)
+        for _ in range(args.steps):
+            tgo.grouped_mmq_pair(x, gate, up, indices, offsets, synth.IQ2_S, 512)
+        torch.cuda.synchronize()
+        kernel_ms, launches = _native.profile_read("forward_gemv")
+        _native.lib.tgo_profile_enable(0)
+        skew_bytes = 57 * 2 * 512 * 8 * 82
+        if launches:
+            report["skewed_256_rows_57_experts"] = {
+                "weight_MB": skew_bytes / 1e6,
+                "kernel_family": _native.lib.tgo_forward_kernel_family(sum(sizes), experts).decode(),
+                "gemv_kernel_us": kernel_ms / launches * 1e3,
+                "GBps_gemv_kernel": skew_bytes / (kernel_ms / launches * 1e-3) / 1e9,
+            }
     for record in report.values():
         rate = record.get("GBps_gemv_kernels", record.get("GBps_gemv_kernel"))
         if rate is not None:
             record["frac_of_hbm_peak"] = rate / PEAK["hbm"]
+            # the north-star target of the decode regime next to what was measured: 0.70 of the HBM peak
+            record["roofline"] = {"bound": "hbm", "achieved": rate, "peak": PEAK["hbm"], "unit": "GB/s",
+                                  "frac": rate / PEAK["hbm"], "target_frac": 0.70,
+                                  "traffic": decode_traffic() if "28672x8192_M1" in str(record.get("name", "")) else None}
     return report
 
 
@@ -346,6 +389,40 @@ def _kernel_us(_native, names):
     return out
 
 
+def measure_dense_cell(args, device, qtype, n, m, k=2048, weight=None) -> dict:
+    """Forward and grad-input kernel time of one dense cell (kernel time from the HIP-event brackets)."""
+    import torch_ggml_ops as tgo
+    import synth
+    from torch_ggml_ops import _native
+
+    if weight is None:
+        weight = synth.random_packed_weight(qtype, (n,), k, 7 + qtype, device=device)
+    generator = torch.Generator(device=device).manual_seed(m)
+    x = torch.randn(m, k, device=device, generator=generator).to(torch.bfloat16)
+    dy = torch.randn(m, n, device=device, generator=generator).to(torch.bfloat16)
+    record = {}
+    for label, fn, kernels in (
+        ("fwd", lambda: tgo.mmq(x, weight, qtype, n), ("quantize", "forward", "forward_gemv")),
+        ("dx", lambda: torch.ops.torch_ggml_ops.mmq_grad_input.default(dy, weight, qtype, k), ("pack_cotangent", "grad_input")),
+    ):
+        for _ in range(args.warmup):
+            fn()
+        torch.cuda.synchronize()
+        _native.lib.tgo_profile_enable(1)
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        times = _kernel_us(_native, kernels)
+        _native.lib.tgo_profile_enable(0)
+        total = sum(times.values())
+        record[label + "_us"] = round(total, 1)
+        record[label + "_TFLOPs"] = round(2.0 * m * n * k / total / 1e6, 1)
+        if m <= 16:
+            record[label + "_weight_GBps"] = round(weight.numel() / total / 1e3, 1)
+    record["forward_operands"] = _native.forward_operand_for(qtype, m, n, 1) if m > 32 else "int8 (GEMV family)"
+    return record
+
+
 def run_dense(args, device) -> None:
     """The dense parity configuration as a sweep: five formats x M in {1, 16, 512, 4096} x N in {2048, 4096},
     K = 2048, forward and grad-input; kernel time per call (quantize + multiply, pack + multiply) and TFLOP/s or,
@@ -362,35 +439,13 @@ def run_dense(args, device) -> None:
         for n in (2048, 4096):
             weight = synth.random_packed_weight(qtype, (n,), k, 7 + qtype, device=device)
             for m in (1, 16, 512, 4096):
-                generator = torch.Generator(device=device).manual_seed(m)
-                x = torch.randn(m, k, device=device, generator=generator).to(torch.bfloat16)
-                dy = torch.randn(m, n, device=device, generator=generator).to(torch.bfloat16)
-                record = {}
-                for label, fn, kernels in (
-                    ("fwd", lambda: tgo.mmq(x, weight, qtype, n), ("quantize", "forward", "forward_gemv")),
-                    ("dx", lambda: torch.ops.torch_ggml_ops.mmq_grad_input.default(dy, weight, qtype, k),
-                     ("pack_cotangent", "grad_input")),
-                ):
-                    for _ in range(args.warmup):
-                        fn()
-                    torch.cuda.synchronize()
-                    _native.lib.tgo_profile_enable(1)
-                    for _ in range(args.steps):
-                        fn()
-                    torch.cuda.synchronize()
-                    times = _kernel_us(_native, kernels)
-                    _native.lib.tgo_profile_enable(0)
-                    total = sum(times.values())
-                    record[label + "_us"] = round(total, 1)
-                    record[label + "_TFLOPs"] = round(2.0 * m * n * k / total / 1e6, 1)
-                    if m <= 16:
-                        record[label + "_weight_GBps"] = round(weight.numel() / total / 1e3, 1)
-                    best = max(best, 2.0 * m * n * k / total / 1e6)
+                record = measure_dense_cell(args, device, qtype, n, m, k, weight)
+                best = max(best, record["fwd_TFLOPs"], record["dx_TFLOPs"])
                 rows_out[f"{qname}_N{n}_M{m}"] = record
     print(json.dumps({
         "metric": "dense mmq forward / grad-input kernel time over the dense parity shapes (value = best TFLOP/s of the sweep)",
         "value": best, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": None, "higher_is_better": True, "dtype": "int8 dot products (forward), bf16 (grad-input), fp32 accumulate",
+        "ms_per_step": None, "higher_is_better": True, "dtype": "int8 or fp16 dot products (forward, per cell), bf16 (grad-input), fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": "dense mmq: Q3_K/Q4_K/Q5_K/Q6_K/IQ2_S x M in {1,16,512,4096} x N in {2048,4096}, K=2048; "
                                "kernel time from HIP-event brackets (launch gaps included)"},
@@ -612,9 +667,10 @@ def main() -> None:
     parser.add_argument("--steps", type=int, default=20)
     parser.add_argument("--warmup", type=int, default=5)
     parser.add_argument("--no-cpu-baseline", action="store_true")
-    parser.add_argument("--decode-cases", default="T1,T4,T8,dense,big",
+    parser.add_argument("--decode-cases", default="T1,T4,T8,dense,big,skewed",
                         help="decode workload: which cases to run (T1, T4, T8: MoE layer calls; dense: Q3_K [4096,2048] "
-                        "single row; big: Q4_K [28672,8192] with 1..16 rows)")
+                        "single row; big: Q4_K [28672,8192] with 1..16 rows; skewed: 256 rows, 200 of them in one of 57 "
+                        "groups, all 256 experts listed)")
     parser.add_argument("--no-sub-records", action="store_true",
                         help="pair workload only: skip the down-projection and decode sub-records")
     parser.add_argument("--workload", choices=("pair", "decode", "multi", "gathered", "layer", "dense", "down"), default="pair")
@@ -734,6 +790,11 @@ def main() -> None:
             breakdown[name].update({"achieved": wk / (breakdown[name]["avg_ms"] * 1e-3), "unit": un, "frac_of_peak": wk / (breakdown[name]["avg_ms"] * 1e-3) / pk})
     if "forward" in breakdown and not half_operands:
         breakdown["forward"]["valu_bound_frac"] = breakdown["forward"]["achieved"] / VALU_BOUND_INT8
+    if args.quant == "Q5_K":
+        # what keeps the two matrix-core kernels from their peak: pipe occupancy from the committed counter runs
+        for name in ("forward", "grad_input"):
+            if name in breakdown:
+                breakdown[name]["pipes"] = measured_pipe_busy(name)
 
     result = {
         "metric": "grouped MMQ pair forward+backward throughput, 256-expert MoE shape",
@@ -775,8 +836,16 @@ def main() -> None:
         decode = measure_decode(args, device)
         result["decode"] = {
             "workload": "T in {1,4,8} x top-8 over 256 experts: gate+up IQ2_S [512,2048] + down Q6_K [2048,512]; "
-                        "dense Q3_K [4096,2048] M=1; dense Q4_K [28672,8192] M=1..16; weight GB/s of the kernels",
+                        "dense Q3_K [4096,2048] M=1; dense Q4_K [28672,8192] M=1..16; 256 rows skewed onto one of 57 "
+                        "experts; weight GB/s of the kernels, each with its roofline block (target 0.70 of HBM)",
             "cases": decode,
+        }
+        # the matrix-core-bound cell of the dense configuration: M = 4096 rows against [4096, 2048], every format
+        result["dense_M4096"] = {
+            "workload": "dense mmq forward / grad-input, x [4096, 2048] x W [4096, 2048]: kernel time and TFLOP/s "
+                        "(peak 2500 for fp16/bf16 operands, 5000 for int8)",
+            "cases": {name: measure_dense_cell(args, device, qtype, 4096, 4096)
+                      for qtype, name in ((11, "Q3_K"), (12, "Q4_K"), (13, "Q5_K"), (14, "Q6_K"), (22, "IQ2_S"))},
         }
     print(json.dumps(result))
 

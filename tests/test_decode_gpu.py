@@ -116,3 +116,33 @@ def test_grouped_decode_skips_invalid_groups(ops, oracle):
     covered = ~np.isnan(exact[:, 0])
     assert covered.sum() == 6
     assert_matches_f32_reference(actual[torch.from_numpy(covered).cuda()], exact[covered])
+
+
+@pytest.mark.parametrize("qname", ("IQ2_S", "Q5_K"))
+def test_skewed_small_batch_listed_with_every_expert(ops, oracle, qname):
+    """256 listed experts, one group of 200 rows and a few single rows: the host sees 256 rows over 256 groups and
+    takes the bandwidth kernel, which walks the large group eight rows at a time (its tasks share the expert's weights
+    through the L2: measured 29 us against 52 us for the matrix-core kernel on the same call with only the non-empty
+    groups listed; one group has to reach about 500 rows before the matrix-core kernel wins, and a call of that many
+    rows over few listed groups takes it anyway).  Results match the oracle either way."""
+    tgo, native, synth = ops
+    qtype, n, k, experts = QTYPES[qname], 96, 512, 256
+    sizes = [0] * experts
+    sizes[7] = 200
+    for expert in (3, 40, 41, 200, 255):
+        sizes[expert] = 1
+    offsets = np.cumsum(sizes).tolist()
+    rows = offsets[-1]
+    assert native.lib.tgo_forward_kernel_family(rows, experts) == b"gemv"
+    host = synth.random_packed_weight(qtype, (experts, n), k, seed=321 + qtype)
+    x = random_bf16((rows, k), seed=12)
+    indices = torch.arange(experts, dtype=torch.int64, device="cuda")
+    actual = tgo.grouped_mmq(x, host.cuda(), indices, torch.tensor(offsets, dtype=torch.int32, device="cuda"), qtype, n)
+    expected = oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), list(range(experts)), offsets, n, k, n)
+    assert_matches_f32_reference(actual, expected)
+    # the same rows with only the non-empty groups listed take the matrix-core kernel
+    listed = [e for e in range(experts) if sizes[e] > 0]
+    assert native.lib.tgo_forward_kernel_family(rows, len(listed)) == b"mfma"
+    compact = tgo.grouped_mmq(x, host.cuda(), torch.tensor(listed, dtype=torch.int64, device="cuda"),
+                              torch.tensor(np.cumsum([sizes[e] for e in listed]).tolist(), dtype=torch.int32, device="cuda"), qtype, n)
+    assert_matches_f32_reference(compact, expected)

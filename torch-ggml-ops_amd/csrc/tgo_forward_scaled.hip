@@ -865,10 +865,6 @@ __global__ __launch_bounds__(64 * FSS_WAVES, 3) void mmq_forward_scaled_short_ke
     // (a wave whose weight rows lie past the end of the matrix repeats the last row and stores nothing: the
     // workgroup's barriers need it)
     const int n0 = tile * FWD_TN + 32 * wave;
-#ifdef FSC_TIMING
-    const unsigned long long t_begin = __builtin_readcyclecounter();
-    const unsigned long long w_begin = wall_clock64();
-#endif
     const int expert = a.task_expert[task];
     const int row_start = a.task_row_start[task];
     const int row_end = a.task_row_end[task];
@@ -1016,9 +1012,6 @@ __global__ __launch_bounds__(64 * FSS_WAVES, 3) void mmq_forward_scaled_short_ke
     park(0);
     publish_rows();
     __syncthreads();
-#ifdef FSC_TIMING
-    const unsigned long long t_loop = __builtin_readcyclecounter();
-#endif
 #pragma unroll 1
     for (int kb = 0; kb < super_blocks; ++kb) {
         const half2_t ratio = {static_cast<_Float16>(incoming.ratio), static_cast<_Float16>(incoming.ratio)};
@@ -1137,15 +1130,6 @@ __global__ __launch_bounds__(64 * FSS_WAVES, 3) void mmq_forward_scaled_short_ke
         __syncthreads();
     }
 
-#ifdef FSC_TIMING
-    const unsigned long long t_done = __builtin_readcyclecounter();
-    if (lane == 0 && wave == 0 && blockIdx.x < 512) {
-        unsigned long long * flat = &fsc_times[0][0][0];
-        flat[3 * blockIdx.x + 0] = t_done - t_begin;
-        flat[3 * blockIdx.x + 1] = wall_clock64();
-        flat[3 * blockIdx.x + 2] = w_begin;
-    }
-#endif
     // ---- epilogue: scale by 2^(E[r] + S[n]) and store 32 rows x 32 columns
     {
         const float row_power = a.row_power[lane_row];

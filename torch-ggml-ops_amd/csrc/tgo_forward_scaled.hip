@@ -120,15 +120,6 @@ constexpr float weight_reach() {
 template <int TYPE>
 constexpr int scale_offset() { return TYPE == Q3_K ? 108 : TYPE == Q6_K ? 208 : 0; }
 
-#ifdef FSC_TIMING
-__device__ unsigned long long fsc_times[8][2][96];
-// phase accumulators in scalar registers; nothing is stored before the end of the kernel
-#define FSC_LAP(slot) do { const unsigned long long now_ = __builtin_readcyclecounter(); lap[slot] += now_ - lap_last; lap_last = now_; } while (0)
-#define FSC_LAP_DUMP(role) do { if (profiled >= 0 && lane == 0) { for (int i_ = 0; i_ < 10; ++i_) fsc_times[profiled][role][i_ + 1 + (wave == FSC_MULTIPLIERS - 1 ? 40 : 0)] = lap[i_]; fsc_times[profiled][role][90] = n_items; fsc_times[profiled][role][94] = wall_clock64() - wall_start; } } while (0)
-#else
-#define FSC_LAP(slot) do {} while (0)
-#define FSC_LAP_DUMP(role) do {} while (0)
-#endif
 
 // Stores the wave's 32 rows x 128 columns of results, which the matrix instructions left transposed (weights as the
 // A operand: the lane holds row l32 and, as element v of tile t, column 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4), as
@@ -220,12 +211,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     if (n_items == 0) {
         return;
     }
-#ifdef FSC_TIMING
-    const int profiled = (wave == 0 || wave == FSC_MULTIPLIERS - 1 || wave == FSC_MULTIPLIERS) && blockIdx.x % 32 == 5 ? blockIdx.x / 32 : -1;
-    unsigned long long lap[10] = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    unsigned long long lap_last = __builtin_readcyclecounter();
-    const unsigned long long wall_start = wall_clock64();
-#endif
     const int super_blocks = a.in_features / QK_K;
     const int total = n_items * super_blocks;   // super-blocks of this workgroup's stream
     auto item_field = [&](int item, int field) {
@@ -561,7 +546,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         }
         publish(&lds.produced[dw], ++written);
         buffer = next_buffer(buffer);
-        FSC_LAP(0);
         int kb = 0;   // of super-block q within its item
 #pragma unroll 1
         for (int q = 0; q < total; ++q) {
@@ -569,7 +553,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             // (past the last super-block the wave works on a repeat of it: nobody reads what that writes)
             // stage 1 of q
             wait_consumed(written + 1 - FSC_BUFFERS);
-            FSC_LAP(1);
             if constexpr (K45) {
                 finish_stage(std::integral_constant<int, 1>{}, inputs, buffer);
             } else {
@@ -580,7 +563,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             if constexpr (K45) {
                 inputs = fetch_inputs(0, parity ^ 1);
             }
-            FSC_LAP(2);
             // stage 0 of q + 1, which may open the next item
             if (kb + 1 == super_blocks) {
                 kb = 0;
@@ -594,9 +576,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             } else {
                 ++kb;
             }
-            FSC_LAP(3);
             wait_consumed(written + 1 - FSC_BUFFERS);
-            FSC_LAP(1);
             if constexpr (K45) {
                 minima_from_header(buffer, inputs.header);
                 finish_stage(std::integral_constant<int, 0>{}, inputs, buffer);
@@ -606,13 +586,10 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             }
             publish(&lds.produced[dw], ++written);
             buffer = next_buffer(buffer);
-            FSC_LAP(4);
             // slot `parity` is free (Q4_K/Q5_K: its last inputs are in registers; the others: stage 1 is done):
             // super-block q + 2 goes there
             advance(parity);
-            FSC_LAP(5);
         }
-        FSC_LAP_DUMP(1);
         return;
     }
 
@@ -723,7 +700,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             stage_as(std::false_type{}, buffer, next_step, ratio);
         }
     };
-    FSC_LAP(0);
     int item = 0, kb = 0;
     int read = 0, buffer = 0;   // stages read so far; stage g is in buffer g % FSC_BUFFERS
     float ratio_next = load_ratio(rows_next, 0);
@@ -741,7 +717,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         const half2_t ratio = {static_cast<_Float16>(ratio_f32), static_cast<_Float16>(ratio_f32)};
         // stage 0; requests stage 1 of the same super-block
         wait_produced(read + 1);
-        FSC_LAP(1);
         stage(buffer, kb * 16 + 8, ratio, active);
         if constexpr (K45) {
             // the super-block's extra reduction step: block minima x block sums (slots 8..15 of the instruction are
@@ -759,7 +734,6 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         }
         publish(&lds.consumed[wave], ++read);
         buffer = next_buffer(buffer);
-        FSC_LAP(2);
         // stage 1; requests stage 0 of the following super-block, which may belong to the next item
         const bool last_of_item = kb + 1 == super_blocks;
         const int item_next = last_of_item ? min(item + 1, n_items - 1) : item;
@@ -767,11 +741,9 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
         rows_next = rows_of(item_next);
         ratio_next = load_ratio(rows_next, kb_next);
         wait_produced(read + 1);
-        FSC_LAP(1);
         stage(buffer, kb_next * 16, ratio, active);
         publish(&lds.consumed[wave], ++read);
         buffer = next_buffer(buffer);
-        FSC_LAP(3);
         if (last_of_item) {
             // The item is complete: scale by 2^(E[r] + S[n]) and store, while the unpacking waves work on the next item.
             const int row_start = item_field(item, 1);
@@ -805,12 +777,10 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             for (int nt = 0; nt < FWD_NT; ++nt) acc[nt] = zero;
             ++item;
             kb = 0;
-            FSC_LAP(4);
         } else {
             ++kb;
         }
     }
-    FSC_LAP_DUMP(0);
 }
 
 // ---- groups of at most 32 rows ---------------------------------------------------------------------------------
@@ -1170,11 +1140,6 @@ __global__ __launch_bounds__(64 * FSS_WAVES, 3) void mmq_forward_scaled_short_ke
     }
 }
 
-#ifdef FSC_TIMING
-extern "C" int tgo_debug_read(void * destination, int bytes) {
-    return static_cast<int>(hipMemcpyFromSymbol(destination, HIP_SYMBOL(fsc_times), bytes));
-}
-#endif
 
 template <int TYPE>
 static hipError_t launch_forward_scaled_typed(const ForwardArgs & call, hipStream_t stream) {

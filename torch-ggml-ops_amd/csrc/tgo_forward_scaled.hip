@@ -53,9 +53,7 @@ constexpr int FSC_STEPS = 8;                                // 16-value reductio
 constexpr int FSC_TILE_BYTES = FWD_NT * FSC_STEPS * 1024;   // fp16 operand of a stage: [tile][step][64 lanes][16 bytes]
 constexpr int FSC_ROWS = 256;                               // activation rows per task
 static_assert(FSC_ROWS == forward_row_tile(12, OPERAND_SCALED), "task rows match the workgroup");
-#ifndef FSC_W_AHEAD
-#define FSC_W_AHEAD 1
-#endif
+constexpr int FSC_W_AHEAD = 1;                               // reduction steps a weight fragment is read ahead of its matrix instructions
 
 constexpr int FSC_MAX_ITEMS = 64;      // items per workgroup (one wave builds the table)
 constexpr int FSC_GRID = 256;          // one workgroup per CU
@@ -594,8 +592,9 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     }
 
     // ---------------- multiplying wave ----------------
-    // Two of these share a SIMD: a lone wave issues a 32 x 32 x 16 matrix instruction only about every 42 cycles,
-    // two keep the pipe close to its 32.
+    // Two of these share a SIMD.  Back-to-back matrix instructions alone issue every 32 cycles from a single wave, but
+    // with the fragment reads and activation requests of this loop in between a lone wave managed one per 42 to 46;
+    // two waves cover each other's waits.
     // Every global address is a uniform 64-bit base, advanced with scalar arithmetic, plus a 32-bit lane offset.
     const int blocks_per_row = a.in_features / 32;
     // Where this wave's 32 activation rows of an item are: a wave without rows in the item reads the workspace's last

@@ -35,6 +35,8 @@ PEAK = {"hbm": 8000.0, "int8": 5000.0, "bf16": 2500.0, "fp32_vector": 157.3}  # 
 # so the vector pipe delivers fp32_vector / 4 lane-operations per second (the published figure counts a fused
 # multiply-add as two and the packed form as two more) and every two of them complete 32 multiply-adds = 64 ops.
 VALU_BOUND_INT8 = PEAK["fp32_vector"] / 4 / 2 * 64  # TOP/s: 1258.4, i.e. 25.2 % of the int8 matrix-core peak
+# Arithmetic type of the forward dot products by the library's operand kind (forward_operand_for).
+OPERAND_DTYPE = {"int8": "int8", "half": "fp16 holding exact integers", "scaled": "fp16 carrying the scales"}
 
 
 def build_pair_workload(device, tokens=8192, experts=256, top_k=8, n=512, k=2048, qtype=13, seed=2024):
@@ -339,11 +341,18 @@ def run_decode(args, device) -> None:
     }))
 
 
+def _native_kind(qtype: int, rows: int, out_features: int, projections: int) -> str:
+    from torch_ggml_ops import _native
+
+    return _native.forward_operand_for(qtype, rows, out_features, projections)
+
+
 def run_multi(args, device) -> None:
     """Several dense projections of one input (attention q/k/v of a GQA layer: 4096 -> 4096, 1024, 1024, Q4_K,
     4096 token rows): three `mmq` calls against one `mmq_multi`, which quantizes the activations once."""
     import torch_ggml_ops as tgo
     import synth
+    from torch_ggml_ops import prepared
 
     rows, k, widths = 4096, 4096, (4096, 1024, 1024)
     generator = torch.Generator(device=device).manual_seed(9)
@@ -372,7 +381,8 @@ def run_multi(args, device) -> None:
         "metric": "dense multi-projection forward throughput (q/k/v of one input, activations quantized once)",
         "value": flops / timings["multi"] / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": timings["multi"] * 1e3, "higher_is_better": True,
-        "dtype": "int8 dot products, fp32 accumulate", "data": "synthetic",
+        "dtype": OPERAND_DTYPE[prepared.multi_operand(qtypes, rows, widths)] + " dot products, fp32 accumulate",
+        "data": "synthetic",
         "config": {"workload": "dense q/k/v: x [4096, 4096] bf16 x Q4_K [4096 | 1024 | 1024, 4096]"},
         "separate_mmq_ms": timings["separate"] * 1e3,
         "speedup_over_separate_calls": timings["separate"] / timings["multi"],
@@ -510,7 +520,8 @@ def run_down(args, device) -> None:
     print(json.dumps({
         "metric": "grouped MMQ down projection fwd+bwd throughput (kernel time)", "value": 2 * flops / both / 1e6,
         "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": both / 1e3,
-        "higher_is_better": True, "dtype": "int8 dot products (forward), bf16 (grad-input), fp32 accumulate",
+        "higher_is_better": True,
+        "dtype": OPERAND_DTYPE[_native_kind(12, rows, 2048, 1)] + " (forward dot products), bf16 (grad-input), fp32 accumulate",
         "data": "synthetic",
         "config": {"workload": f"grouped_mmq fwd+bwd: 256 experts, down Q4_K [2048,512], T=4096 x top-8 ({rows} rows), "
                                "Zipf-skewed routing; three weight copies in turn"},
@@ -555,7 +566,7 @@ def run_gathered(args, device) -> None:
         "metric": "grouped gate+up forward throughput from unsorted token activations (gather folded into the quantizer)",
         "value": flops / timings["gathered"] / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": timings["gathered"] * 1e3, "higher_is_better": True,
-        "dtype": "int8 dot products, fp32 accumulate", "data": "synthetic",
+        "dtype": OPERAND_DTYPE[_native_kind(13, rows, n, 2)] + " dot products, fp32 accumulate", "data": "synthetic",
         "config": {"workload": f"grouped_mmq_pair forward: 256 experts, gate+up Q5_K [512,2048], T=8192 x top-8 ({rows} rows), "
                                "token activations [8192, 2048] + int64 row index"},
         "index_select_then_pair_ms": timings["index_select"] * 1e3,
@@ -748,7 +759,7 @@ def main() -> None:
     operand_kind = _native.forward_operand_for(w["qtype"], rows, n, 2)
     half_operands = operand_kind in ("half", "scaled")
     forward_peak = PEAK["bf16"] if half_operands else PEAK["int8"]   # fp16 and bf16 share the dense matrix peak
-    forward_dtype = {"int8": "int8", "half": "fp16 holding exact integers", "scaled": "fp16 carrying the scales"}[operand_kind]
+    forward_dtype = OPERAND_DTYPE[operand_kind]
     # bytes the quantizer moves: bf16 in; int8 or fp16 values, an fp32 scale and sum per 32 values, and for the scaled
     # operands a power of two and eight fp16 block sums per 256 values and a power of two per row out
     quantize_bytes = rows * k * 2 + rows * k * (2 if half_operands else 1) + 2 * rows * (k // 32) * 4

@@ -110,6 +110,19 @@ int tgo_mmq_forward_prepared(const void * workspace, const void * packed, void *
                              int64_t rows, int64_t in_features, int64_t out_features,
                              int quant_type, void * stream);
 
+/* tgo_quantize_q8_1 and tgo_mmq_forward_prepared for a caller that names the operand kind itself
+ * (TGO_OPERAND_INT8, TGO_OPERAND_HALF or TGO_OPERAND_SCALED, see tgo_set_forward_operand) instead of
+ * leaving it to the setting: a caller that knows every projection it will run on the workspace
+ * asks tgo_forward_operand_for with their summed out_features and passes the answer to both, which
+ * gives several large projections of one input the scaled kernels that a single large call gets.
+ * Both calls must name the same kind; outputs turn into NaN when they do not.  No counterpart in
+ * the reference. */
+int tgo_quantize_q8_1_as(const void * input_bf16, void * workspace, int64_t rows, int64_t in_features,
+                         int operand, void * stream);
+int tgo_mmq_forward_prepared_as(const void * workspace, const void * packed, void * output_bf16,
+                                int64_t rows, int64_t in_features, int64_t out_features,
+                                int quant_type, int operand, void * stream);
+
 /* Bytes of the workspace of the grad-input entry points: the cotangent(s) copied into MFMA
  * fragment order (rows padded to 32, columns to 16), preceded by the task list when
  * num_groups > 0.  `sources` is 1, or 2 for the fused pair; num_groups is 0 for the dense call.
@@ -259,7 +272,7 @@ int tgo_profile_read(int kernel, double * total_ms, int64_t * launches);
  *                       a grouped call; both projections of a pair count), otherwise fp16 for IQ2_S (whose integer
  *                       operand needs two int8 planes but one fp16 number) and int8 for the other formats.
  * Workspaces that are quantized before their format is known (tgo_quantize_q8_1 / tgo_mmq_forward_prepared) take int8
- * unless TGO_OPERAND_HALF is forced.  The activation workspace is laid out for one kind and says which in its last
+ * unless TGO_OPERAND_HALF is forced (their _as variants take the kind as an argument).  The activation workspace is laid out for one kind and says which in its last
  * KiB: tgo_q8_workspace_unpack follows that tag, and tgo_mmq_forward_prepared turns its outputs into NaN when the
  * setting was changed between quantizing a workspace and using it.  A call reads the setting once.
  * tgo_forward_operand() returns the current setting; tgo_forward_operand_for() the kind (never AUTO) that a forward

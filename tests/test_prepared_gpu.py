@@ -12,7 +12,7 @@ int8 operands forced (and by default for the other formats); under the default t
 import pytest
 import torch
 
-from helpers import QTYPES, assert_matches_f32_reference, bits, random_bf16
+from helpers import OPERAND_NOISE, QTYPES, assert_matches_f32_reference, bits, random_bf16
 
 pytestmark = pytest.mark.gpu
 
@@ -87,6 +87,48 @@ def test_multi_projection_forward_and_gradient(ops, operand):
     first.backward(grads[0])
     only = torch.ops.torch_ggml_ops.mmq_grad_input.default(grads[0], weights[0], qtypes[0], k)
     torch.testing.assert_close(z.grad, only, rtol=0, atol=0)
+
+
+@pytest.mark.parametrize("kind", ("int8", "half", "scaled"))
+def test_workspace_of_a_named_kind_matches_the_oracle(ops, oracle, kind):
+    """A caller may name the operand kind of a workspace: every format's kernel of that kind reads it."""
+    tgo, synth = ops
+    rows, k = 300, 1024
+    x = random_bf16((rows, k), seed=17)
+    workspace = tgo.quantize_q8_1(x, operand=kind)
+    for qname, n in (("Q4_K", 96), ("Q6_K", 37), ("IQ2_S", 160), ("Q5_K", 512), ("Q3_K", 64)):
+        qtype = QTYPES[qname]
+        host = synth.random_packed_weight(qtype, (n,), k, seed=900 + qtype)
+        prepared = tgo.mmq_prepared(workspace, host.cuda(), rows, k, qtype, n, operand=kind)
+        assert_matches_f32_reference(prepared, oracle.mmq_forward(qtype, bits(x), host.numpy(), n, k),
+                                     accumulate_noise=OPERAND_NOISE[kind])
+    # the same workspace read as another kind: refused on the device, every output NaN
+    other = "int8" if kind != "int8" else "scaled"
+    weight = synth.random_packed_weight(12, (64,), k, seed=5).cuda()
+    assert torch.isnan(tgo.mmq_prepared(workspace, weight, rows, k, 12, 64, operand=other).float()).all()
+    with pytest.raises(ValueError, match="operand must be"):
+        tgo.quantize_q8_1(x, operand="fp8")
+
+
+def test_multi_projection_of_a_long_sequence_takes_the_scaled_kernels(ops):
+    """q/k/v of 2048 rows fill the chip together: mmq_multi quantizes for, and runs, the scaled kernels, and each
+    projection agrees with a separate mmq (scaled or int8 by its own size) within the scaled kind's rounding."""
+    from torch_ggml_ops import prepared
+
+    tgo, synth = ops
+    rows, k, widths = 2048, 512, (2048, 1024, 1024)
+    qtypes = [QTYPES["Q4_K"], QTYPES["Q4_K"], QTYPES["Q6_K"]]
+    assert prepared.multi_operand(qtypes, rows, widths) == "scaled"
+    assert prepared.multi_operand(qtypes, 40, widths) == "int8"
+    assert prepared.multi_operand([QTYPES["IQ2_S"]] * 2, 40, widths[:2]) == "half"
+    assert prepared.multi_operand([QTYPES["IQ2_S"], QTYPES["Q4_K"]], 40, widths[:2]) == "int8"
+    weights = [synth.random_packed_weight(q, (n,), k, seed=60 + i).cuda() for i, (q, n) in enumerate(zip(qtypes, widths))]
+    x = random_bf16((rows, k), seed=9)
+    outputs = tgo.mmq_multi(x, weights, qtypes, widths)
+    for output, weight, qtype, n in zip(outputs, weights, qtypes, widths):
+        plain = tgo.mmq(x, weight, qtype, n).float()
+        tolerance = plain.abs() * 2.0**-7 + 2 * OPERAND_NOISE["scaled"] * float(plain.abs().max())
+        assert bool(((output.float() - plain).abs() <= tolerance).all())
 
 
 def test_prepared_rejects_mismatched_workspace(ops):

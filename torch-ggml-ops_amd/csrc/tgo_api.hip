@@ -282,15 +282,29 @@ int tgo_dequant_bf16(const void * packed, void * out_bf16, int64_t rows, int64_t
                      "dequant_bf16 launch");
 }
 
-int tgo_quantize_q8_1(const void * input_bf16, void * workspace, int64_t rows, int64_t in_features,
-                      void * stream) {
+static int check_workspace_operand(int operand) {
+    if (operand != TGO_OPERAND_INT8 && operand != TGO_OPERAND_HALF && operand != TGO_OPERAND_SCALED) {
+        return fail(TGO_ERR_INVALID,
+                    "a workspace holds TGO_OPERAND_INT8, TGO_OPERAND_HALF or TGO_OPERAND_SCALED operands; got %d", operand);
+    }
+    return TGO_OK;
+}
+
+int tgo_quantize_q8_1_as(const void * input_bf16, void * workspace, int64_t rows, int64_t in_features, int operand,
+                         void * stream) {
     TGO_TRY(check_matmul_shape(rows, in_features, 1, TGO_TYPE_Q4_K));
     TGO_TRY(check_pointer(input_bf16, "input"));
     TGO_TRY(check_pointer(workspace, "workspace"));
-    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(0));
+    TGO_TRY(check_workspace_operand(operand));
+    const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0), operand);
     return check_hip(tgo::launch_quantize_q8_1(static_cast<const uint16_t *>(input_bf16), view, rows, in_features,
                                                static_cast<hipStream_t>(stream)),
                      "quantize_q8_1 launch");
+}
+
+int tgo_quantize_q8_1(const void * input_bf16, void * workspace, int64_t rows, int64_t in_features,
+                      void * stream) {
+    return tgo_quantize_q8_1_as(input_bf16, workspace, rows, in_features, tgo::forward_operand_kind(0), stream);
 }
 
 int tgo_q8_workspace_unpack(const void * workspace, void * q_int8, void * d_f32, void * sum_f32,
@@ -348,25 +362,32 @@ int tgo_mmq_forward_static(const void * input_bf16, const void * packed, void * 
                            stream);
 }
 
-int tgo_mmq_forward_prepared(const void * workspace, const void * packed, void * output_bf16, int64_t rows,
-                             int64_t in_features, int64_t out_features, int quant_type, void * stream) {
+int tgo_mmq_forward_prepared_as(const void * workspace, const void * packed, void * output_bf16, int64_t rows,
+                                int64_t in_features, int64_t out_features, int quant_type, int operand, void * stream) {
     TGO_TRY(check_matmul_shape(rows, in_features, out_features, quant_type));
     TGO_TRY(check_pointer(workspace, "workspace"));
     TGO_TRY(check_pointer(packed, "packed_weight"));
     TGO_TRY(check_pointer(output_bf16, "output"));
+    TGO_TRY(check_workspace_operand(operand));
     const tgo::Q8Workspace view =
-        tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), tgo::forward_operand_kind(0));
+        tgo::q8_workspace_view(const_cast<void *>(workspace), rows, in_features, tgo::use_gemv(rows, 0), operand);
     const auto launch = tgo::use_gemv(rows, 0) ? tgo::launch_mmq_gemv : tgo::launch_mmq_forward;
     TGO_TRY(check_hip(launch(static_cast<const uint8_t *>(packed), nullptr, 0, view,
                              static_cast<uint16_t *>(output_bf16), nullptr, nullptr, static_cast<int>(rows),
                              static_cast<int>(in_features), static_cast<int>(out_features), quant_type,
                              static_cast<hipStream_t>(stream)),
                       "mmq_forward_prepared launch"));
-    // (the workspace was quantized by an earlier call: had the operand setting changed in between, its layout would
-    // not be the one this launch assumed)
+    // (the workspace was quantized by an earlier call: were it of another kind than this call was told, its layout
+    // would not be the one this launch assumed)
     return check_hip(tgo::launch_workspace_guard(view, static_cast<uint16_t *>(output_bf16), rows * out_features,
                                                  static_cast<hipStream_t>(stream)),
                      "workspace guard launch");
+}
+
+int tgo_mmq_forward_prepared(const void * workspace, const void * packed, void * output_bf16, int64_t rows,
+                             int64_t in_features, int64_t out_features, int quant_type, void * stream) {
+    return tgo_mmq_forward_prepared_as(workspace, packed, output_bf16, rows, in_features, out_features, quant_type,
+                                       tgo::forward_operand_kind(0), stream);
 }
 
 int tgo_mmq_grad_input(const void * grad_output_bf16, const void * packed, void * grad_input_bf16,

@@ -37,6 +37,8 @@ lib.tgo_q8_workspace_unpack.argtypes = [_p, _p, _p, _p, _i64, _i64, _p]
 lib.tgo_mmq_forward.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_mmq_forward_static.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_mmq_forward_prepared.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _p]
+lib.tgo_quantize_q8_1_as.argtypes = [_p, _p, _i64, _i64, _int, _p]
+lib.tgo_mmq_forward_prepared_as.argtypes = [_p, _p, _p, _i64, _i64, _i64, _int, _int, _p]
 lib.tgo_grad_workspace_bytes.argtypes = [_i64, _i64, _i64, _int]
 lib.tgo_grad_workspace_bytes.restype = _i64
 lib.tgo_dense_grad_workspace_bytes.argtypes = [_i64, _i64, _i64, _int]
@@ -74,6 +76,8 @@ EXPORTS = (
     "tgo_mmq_forward",
     "tgo_mmq_forward_static",
     "tgo_mmq_forward_prepared",
+    "tgo_quantize_q8_1_as",
+    "tgo_mmq_forward_prepared_as",
     "tgo_mmq_grad_input",
     "tgo_grouped_mmq_forward",
     "tgo_grouped_mmq_forward_gathered",

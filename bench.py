@@ -663,7 +663,8 @@ def run_layer(args, device) -> None:
         "metric": "SwiGLU MoE layer forward throughput, token activations in, token outputs out",
         "value": flops / elapsed / 1e12, "unit": "TFLOP/s", "n_gpus": 1, "steps": args.steps,
         "warmup": args.warmup, "ms_per_step": elapsed * 1e3, "higher_is_better": True,
-        "dtype": "int8 dot products, fp32 accumulate", "data": "synthetic",
+        "dtype": OPERAND_DTYPE[_native_kind(qtype, rows, intermediate, 2)] + " dot products, fp32 accumulate",
+        "data": "synthetic",
         "config": {"workload": f"moe_layer forward: 256 experts, gate/up/down Q5_K, features 2048, intermediate 512, "
                                f"T=8192 x top-8 ({rows} sorted rows)"},
         "kernels": kernels,

@@ -178,8 +178,10 @@ int tgo_grouped_mmq_forward_gathered(const void * input_bf16, const int64_t * ro
 /* Gate/up pair with the SwiGLU activation fused into the epilogue: output_gate[rows, out_features] is the
  * first projection as tgo_grouped_mmq_forward writes it, output_activated[rows, out_features] is
  * bf16( silu(gate) * up ) with gate and up rounded to bf16 first, i.e. what the caller-side
- * silu(gate) * up computes from the pair's outputs, up to one rounding less.  The up projection is never
- * written, and no activation kernel re-reads the pair.  `row_index` may be NULL (rows are input rows) or the
+ * silu(gate) * up computes from the pair's outputs, up to one rounding less.  With int8 or exact fp16
+ * operands the up projection is never written and no activation kernel re-reads the pair; with the scaled
+ * operands of large calls the up projection passes through output_activated and an elementwise launch
+ * replaces it (same values; still faster than the other kinds at that size).  `row_index` may be NULL (rows are input rows) or the
  * gather index of tgo_grouped_mmq_forward_gathered.  Same workspace as tgo_grouped_mmq_forward.  Always runs
  * the MFMA kernel family.  No counterpart in the reference, whose pair operator returns both projections
  * (grouped_mmq_pair_cuda, csrc/mmq_hip.cu:1054-1193) and leaves the activation to the caller. */
@@ -266,8 +268,9 @@ int tgo_profile_read(int kernel, double * total_ms, int64_t * launches);
  *                       activation and the dequantized weight, each normalised by a power of two per row and rounded
  *                       to fp16 once (relative 2^-11; same quants, block scales and sums as the other kinds).  Results
  *                       differ from the other kinds by up to 5e-4 of the largest output; the fastest kind for calls
- *                       that fill the chip.  The fused SwiGLU entry point has no such kernel and takes int8 (fp16 for
- *                       IQ2_S) when this kind is forced.
+ *                       that fill the chip.  Its kernel has no SwiGLU epilogue: tgo_grouped_mmq_swiglu then stores both
+ *                       projections and finishes with an elementwise pass (same results as the pair followed by
+ *                       silu(gate) * up on the bf16 values).
  *   TGO_OPERAND_AUTO    (default) scaled for calls of at least 128 tiles of 256 rows x 128 outputs (total rows of
  *                       a grouped call; both projections of a pair count), otherwise fp16 for IQ2_S (whose integer
  *                       operand needs two int8 planes but one fp16 number) and int8 for the other formats.

@@ -67,9 +67,20 @@ def test_fused_activation_against_the_oracle(ops, oracle, qname):
     assert max_rel_to_peak(f32(activated), expected) < 1e-2
 
 
+@pytest.fixture(params=("auto", "scaled"))
+def operand(request):
+    """"scaled": the kind that large calls take by themselves, whose kernel stores both projections and leaves the
+    activation to an elementwise pass; forced here so that the small shapes below reach it."""
+    from torch_ggml_ops import _native
+
+    _native.set_forward_operand(request.param)
+    yield request.param
+    _native.set_forward_operand("auto")
+
+
 @pytest.mark.parametrize("qname", tuple(QTYPES))
 @pytest.mark.parametrize("n", (512, 96, 37))
-def test_fused_activation_matches_pair_then_swiglu(ops, qname, n):
+def test_fused_activation_matches_pair_then_swiglu(ops, operand, qname, n):
     """n = 512: whole tiles; 96: a partial column tile; 37: odd row stride, element-wise stores."""
     tgo, synth = ops
     qtype, k = QTYPES[qname], 512
@@ -86,7 +97,7 @@ def test_fused_activation_matches_pair_then_swiglu(ops, qname, n):
     torch.testing.assert_close(tgo.grouped_mmq_swiglu(x, gate_w, up_w, *metadata, qtype, n), activated, rtol=0, atol=0)
 
 
-def test_fused_activation_from_token_rows(ops):
+def test_fused_activation_from_token_rows(ops, operand):
     tgo, synth = ops
     qtype, n, k, tokens, top_k, experts = 13, 256, 1024, 120, 4, 8
     gate_w = synth.random_packed_weight(qtype, (experts, n), k, seed=41).cuda()

@@ -439,15 +439,14 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
     const int64_t bytes_per_expert = out_features * (in_features / tgo::QK_K) * tgo::block_bytes(quant_type);
     // (the fused SwiGLU epilogue exists in the MFMA kernel only)
     const bool gemv = !swiglu && tgo::use_gemv(rows, num_groups);
-    // (the scaled-operand kernel has no fused SwiGLU epilogue)
-    int operand_kind = tgo::forward_operand_kind(quant_type, rows, out_features, packed_second != nullptr ? 2 : 1);
-    if (swiglu && operand_kind == tgo::OPERAND_SCALED) {
-        operand_kind = quant_type == TGO_TYPE_IQ2_S ? tgo::OPERAND_HALF : tgo::OPERAND_INT8;
-    }
+    const int operand_kind = tgo::forward_operand_kind(quant_type, rows, out_features, packed_second != nullptr ? 2 : 1);
+    // the scaled-operand kernel has no SwiGLU epilogue: it stores both projections (the up projection where the
+    // result goes) and an elementwise pass finishes, which costs less than the other kinds' kernels lose to it
+    const bool fused = swiglu && operand_kind != tgo::OPERAND_SCALED;
     const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, gemv, operand_kind);
     void * task_base = static_cast<char *>(workspace) + (tgo::q8_workspace_bytes(rows, in_features) + 15) / 16 * 16;
     const int row_tile = gemv ? tgo::GEMV_ROW_TILE : tgo::forward_row_tile(quant_type, view.operand_kind());
-    const auto launch = swiglu ? tgo::launch_mmq_forward_swiglu : gemv ? tgo::launch_mmq_gemv : tgo::launch_mmq_forward;
+    const auto launch = fused ? tgo::launch_mmq_forward_swiglu : gemv ? tgo::launch_mmq_gemv : tgo::launch_mmq_forward;
     const tgo::TaskList tasks = tgo::task_list_view(task_base, rows, num_groups, row_tile);
 
     // the quantizer writes the tile-task list on the side; the MFMA kernel runs a task of at most 32 rows in
@@ -464,6 +463,11 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
                              static_cast<uint16_t *>(output_second), &tasks, static_cast<int>(rows),
                              static_cast<int>(in_features), static_cast<int>(out_features), quant_type, hip_stream),
                       "grouped mmq_forward launch"));
+    if (swiglu && !fused) {
+        TGO_TRY(check_hip(tgo::launch_swiglu_rows(static_cast<const uint16_t *>(output_first),
+                                                  static_cast<uint16_t *>(output_second), rows * out_features, hip_stream),
+                          "swiglu launch"));
+    }
     return TGO_OK;
 }
 

@@ -234,3 +234,69 @@ def test_prepared_forward_refuses_a_workspace_of_another_kind(ops):
         assert torch.isnan(out).all()
     finally:
         native.set_forward_operand("auto")
+
+
+@pytest.mark.parametrize("seed", range(10))
+def test_ragged_groups_of_any_mix_under_the_scaled_kind(ops, oracle, seed):
+    """Seeded random group lists for the two kernels of the scaled kind: empty groups, whole groups of at most 32 rows
+    (their own kernel, listed behind the others), groups that end a few rows into a 256-row tile, repeated and
+    unsorted experts, column counts off the 128-column tile and off the 16-byte stores, one or two projections."""
+    tgo, native, synth = ops
+    rng = np.random.default_rng(9000 + seed)
+    qtype = list(QTYPES.values())[seed % len(QTYPES)]
+    n = int(rng.choice([37, 128, 200, 264]))
+    k = int(rng.choice([256, 768, 1024]))
+    experts_total = 16
+    groups = int(rng.integers(5, 14))
+    sizes = rng.choice([0, 1, 2, 31, 32, 33, 64, 255, 256, 257, 300, 520], size=groups).tolist()
+    if sum(sizes) == 0:
+        sizes[0] = 40
+    experts = rng.integers(0, experts_total, size=groups).tolist()
+    offsets = np.cumsum(sizes).tolist()
+    first_host = synth.random_packed_weight(qtype, (experts_total, n), k, seed=100 + seed)
+    second_host = synth.random_packed_weight(qtype, (experts_total, n), k, seed=200 + seed)
+    x = random_bf16((offsets[-1], k), seed=300 + seed)
+    metadata = _metadata(experts, offsets)
+    native.set_forward_operand("scaled")
+    try:
+        if seed % 2 == 0:
+            first, second = tgo.grouped_mmq_pair(x, first_host.cuda(), second_host.cuda(), *metadata, qtype, n)
+        else:
+            first, second = tgo.grouped_mmq(x, first_host.cuda(), *metadata, qtype, n), None
+    finally:
+        native.set_forward_operand("auto")
+    expected = oracle.grouped(oracle.mmq_forward, qtype, bits(x), first_host.numpy(), experts, offsets, n, k, n)
+    assert_matches_f32_reference(first, expected, OPERAND_NOISE["scaled"])
+    if second is not None:
+        expected = oracle.grouped(oracle.mmq_forward, qtype, bits(x), second_host.numpy(), experts, offsets, n, k, n)
+        assert_matches_f32_reference(second, expected, OPERAND_NOISE["scaled"])
+
+
+@pytest.mark.parametrize("grouped", (False, True))
+def test_more_tiles_than_one_table_per_cu_holds(ops, grouped):
+    """16 384 rows x 32 896 outputs: 64 row tasks x 257 column tiles, more than the 64 items that each of the 256
+    workgroups of the scaled kernel keeps in its table, so the launch grows its grid.  Checked against the int8 kind
+    (itself pinned on the oracle at the sizes the oracle finishes)."""
+    tgo, native, synth = ops
+    qtype, rows, n, k = QTYPES["Q4_K"], 16384, 32896, 256
+    weight = synth.random_packed_weight(qtype, (4, n) if grouped else (n,), k, seed=77).cuda()
+    x = random_bf16((rows, k), seed=78)
+    metadata = _metadata([1, 3, 0], [5000, 5020, rows])
+
+    def run():
+        return tgo.grouped_mmq(x, weight, *metadata, qtype, n) if grouped else tgo.mmq(x, weight, qtype, n)
+
+    assert native.forward_operand_for(qtype, rows, n) == "scaled"
+    scaled = run()
+    native.set_forward_operand("int8")
+    try:
+        exact = run()
+    finally:
+        native.set_forward_operand("auto")
+    peak = float(exact.float().abs().max())
+    step = 1 << 22   # (compared in slices: the fp32 copies of a gigabyte of bf16 would be four)
+    flat_scaled, flat_exact = scaled.view(-1), exact.view(-1)
+    for begin in range(0, flat_exact.numel(), step * 16):
+        a = flat_scaled[begin : begin + step * 16].float()
+        b = flat_exact[begin : begin + step * 16].float()
+        assert bool(((a - b).abs() <= b.abs() * 2.0**-7 + OPERAND_NOISE["scaled"] * peak).all())

@@ -156,7 +156,8 @@ def test_pair_and_fused_swiglu(ops, oracle, operand, qname):
     with np.errstate(over="ignore"):
         expected = gate_bf16 / (1.0 + np.exp(-gate_bf16)) * up_ref.astype(np.float64)
     assert nrmse(f32(activated), expected) < 5e-3
-    assert max_rel_to_peak(f32(activated), expected) < 1e-2
+    # (the scaled kind's operand rounding reaches both factors of the product)
+    assert max_rel_to_peak(f32(activated), expected) < (1.5e-2 if operand == "scaled" else 1e-2)
 
 
 @pytest.mark.parametrize("qname", tuple(QTYPES))

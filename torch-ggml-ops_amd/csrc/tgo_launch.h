@@ -225,9 +225,9 @@ hipError_t launch_dequant_bf16(const uint8_t * packed, uint16_t * out, int64_t r
 hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, int64_t rows,
                                 int64_t in_features, hipStream_t stream, const int64_t * gather = nullptr,
                                 int64_t input_rows = 0, const TaskBuild * build = nullptr);
-// Turns `count` bf16 outputs into NaN when the workspace's tag is not the layout of `ws` (runs behind the multiply kernel).
 // up_then_activated[i] = swiglu(gate[i], up_then_activated[i]) over `count` bf16 values (timed with the forward kernels).
 hipError_t launch_swiglu_rows(const uint16_t * gate, uint16_t * up_then_activated, int64_t count, hipStream_t stream);
+// Turns `count` bf16 outputs into NaN when the workspace's tag is not the layout of `ws` (runs behind the multiply kernel).
 hipError_t launch_workspace_guard(const Q8Workspace & ws, uint16_t * out, int64_t count, hipStream_t stream);
 hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float * sum, int64_t rows,
                             int64_t in_features, hipStream_t stream);

@@ -615,6 +615,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     if (tasks != nullptr) {
         args.task_count = tasks->count;
         args.task_early = tasks->early;
+        args.task_cursor = tasks->cursor;
         args.task_expert = tasks->expert;
         args.task_row_start = tasks->row_start;
         args.task_row_end = tasks->row_end;
@@ -623,6 +624,7 @@ static hipError_t launch_forward(const uint8_t * packed, const uint8_t * packed_
     } else {
         args.task_count = nullptr;
         args.task_early = nullptr;
+        args.task_cursor = nullptr;
         args.task_expert = nullptr;
         args.task_row_start = nullptr;
         args.task_row_end = nullptr;

@@ -26,6 +26,7 @@ struct ForwardArgs {
     uint16_t * y_second;
     const int32_t * task_count;   // nullptr: dense
     const int32_t * task_early;   // tasks listed before those of at most 32 rows
+    int32_t * task_cursor;        // zero at launch; counts the short items that workgroups have taken
     const int32_t * task_expert;
     const int32_t * task_row_start;
     const int32_t * task_row_end;

@@ -32,11 +32,15 @@
 // the time.)  LDS executes a wave's accesses in issue order, so a counter written after the data, or after the
 // last read, needs no wait of its own.
 //
-// A workgroup is persistent: it owns every gridDim.x-th (task, column tile) item of the launch and runs their
-// super-blocks as one stream, so an item's first loads (task description, packed blocks, the scan of its scales,
+// A workgroup is persistent: it owns every n-th (task, column tile) item of the launch, n being the number of role-split
+// workgroups (one per CU), and runs their super-blocks as one stream, so an item's first loads (task description, packed blocks, the scan of its scales,
 // activation fragments) are requested while the item before it is still being multiplied, and its results are
 // stored while the unpackers already work on the next one.  With one item per workgroup those latencies and the
 // epilogue, none of them overlapped by anything on a CU that holds a single workgroup, were 40 % of the kernel's time.
+//
+// Grouped calls keep their groups of at most 32 rows out of these workgroups: the launch ends in workgroups that run
+// short_group_items() on them instead (below), and which the CUs take up as their role-split workgroup runs out of
+// items: the last round of role-split items occupies a fraction of the CUs only.
 #include <type_traits>
 
 #include "tgo_device.h"
@@ -161,12 +165,417 @@ TGO_DEVICE void store_rows_32x128(const v16f (&tiles)[FWD_NT], uint16_t * dst, i
     }
 }
 
+// ---- groups of at most 32 rows ---------------------------------------------------------------------------------
+// A task of a few rows costs the role-split workgroups below what a full one costs their unpacking waves, while seven of
+// their eight multiplying waves have nothing to do: on a routing with many small groups a third of the time went into
+// 1.5 % of the rows.  Such tasks (the list keeps whole groups of at most 32 rows behind the others) go to workgroups of
+// the same launch that run this routine instead, in which every wave unpacks: a wave owns 32 weight rows of the task's column tile and the task's one 32-row activation
+// tile, from the packed blocks to the stored results, and never meets another wave.  Its fp16 weights stay in
+// registers: the lane that unpacks k-half h of a 32-value block of weight row n holds exactly the two matrix-instruction
+// fragments of reduction step 2 * block + h, and one exchange between the half-waves (v_permlane32_swap) per register
+// puts them where the instruction wants them.  Three such groups of four waves make a workgroup, so that twelve waves keep
+// the vector pipe busy where four did.  The algebra is that of the role-split routine except for the weight normalisation,
+// which is per super-block here (see below): the two agree to fp32 rounding of that last step, not bit for bit.
+constexpr int FSS_WAVES = 4;
+
+template <int TYPE>
+struct ShortLds {
+    static constexpr int RAW_SLOT = ScaledLds<TYPE>::RAW_SLOT;
+    alignas(16) uint8_t raw[FSS_WAVES][32 * RAW_SLOT];   // per wave: the packed blocks of one super-block
+    alignas(16) uint8_t x[16 * 1024];                    // the task's activation fragments of one super-block
+    alignas(16) float column_power[FSS_WAVES][32];       // 2^s of the wave's weight rows in the current super-block
+    alignas(16) int arrived[FSS_WAVES];                  // barriers of the group that each of its waves has reached
+    int next_item;                                       // the item that the group has taken from the list
+    std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;
+};
+
+// `tid`: the thread's index in its group of FSS_WAVES waves; `group`: which of the groups that share the workgroup
+// this is; `blocks` workgroups run short items.  The groups of a workgroup run side by side like workgroups of their
+// own: what one waits for (its packed blocks, its barrier) the others cover with their unpacking, which they could not
+// if the workgroup's barrier held them in step.  So a group synchronises its four waves through counters in LDS (LDS
+// executes a wave's accesses in issue order: a count written after the data, or after the last read, needs no wait of
+// its own), and takes its items from the list's cursor by itself.  Three groups that unpack side by side on a CU each
+// take more than twice as long as one that is alone there, so towards the end of the list the later groups stop
+// taking items and the last ones are spread over the CUs.  Workgroups that start late, on the CUs of the role-split
+// workgroups that ran longest, simply take fewer.
 template <int TYPE, bool WIDE>
-__global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(const ForwardArgs a, const int total_slots) {
+TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, const int tid, const int group, const int blocks) {
+    using F = Format<TYPE>;
+    constexpr bool K45 = TYPE == Q4_K || TYPE == Q5_K;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int l32 = lane & 31;
+    const int half = lane >> 5;
+    if constexpr (TYPE == IQ2_S) {
+        expand_iq2s_selectors(lds.codebook, tid, 64 * FSS_WAVES);
+    }
+    if (tid < FSS_WAVES) {
+        lds.arrived[tid] = 0;
+    }
+    __syncthreads();   // (of the whole workgroup: its groups are still in step here, and part ways behind it)
+    static_assert(FSS_WAVES == 4, "one 16-byte read covers the group's counters");
+    typedef int i32x4_t __attribute__((ext_vector_type(4)));
+    int barriers_passed = 0;
+    auto group_barrier = [&]() __attribute__((always_inline)) {
+        ++barriers_passed;
+        asm volatile("" ::: "memory");   // (the data accesses stay before the count)
+        if (lane == 0) {
+            *(volatile __attribute__((address_space(3))) int *)&lds.arrived[wave] = barriers_passed;
+        }
+        for (int polls = 0; polls < FSC_SPIN_LIMIT; ++polls) {
+            const i32x4_t v = *(const volatile __attribute__((address_space(3))) i32x4_t *)&lds.arrived[0];
+            if (__builtin_amdgcn_readfirstlane(min(min(v.x, v.y), min(v.z, v.w))) >= barriers_passed) {
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        asm volatile("" ::: "memory");   // (the data accesses stay after the count)
+    };
+    // The number of short tasks is known on the device only (one round trip to read it).
+    const int inner = a.n_tiles * a.projections;
+    const int tasks = a.task_count[0];
+    const int first_short = min(a.task_early[0], tasks);
+    const int items = (tasks - first_short) * inner;
+#pragma unroll 1
+    for (;;) {
+    if (tid == 0) {
+        // (an estimate of what is left decides whether this group still takes part; the count itself is exact)
+        const int left = items - __hip_atomic_load(a.task_cursor, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        // (a group's first item: while any is left -- the groups that started with it are all busy as long; later: only
+        // if the groups before it, one more item each, would not finish the list)
+        const int taken = left > (barriers_passed == 0 ? 0 : group * blocks) ? atomicAdd(a.task_cursor, 1) : items;
+        *(volatile __attribute__((address_space(3))) int *)&lds.next_item = taken;
+    }
+    group_barrier();
+    const int item = __builtin_amdgcn_readfirstlane(*(const volatile __attribute__((address_space(3))) int *)&lds.next_item);
+    if (item >= items) {
+        break;
+    }
+    const int task = first_short + item / inner;
+    int tile = item % inner;
+    const bool second = tile >= a.n_tiles;
+    tile -= second ? a.n_tiles : 0;
+    // (a wave whose weight rows lie past the end of the matrix repeats the last row and stores nothing: the
+    // workgroup's barriers need it)
+    const int n0 = tile * FWD_TN + 32 * wave;
+    const int expert = a.task_expert[task];
+    const int row_start = a.task_row_start[task];
+    const int row_end = a.task_row_end[task];
+    const int super_blocks = a.in_features / QK_K;
+    const int blocks_per_row = a.in_features / 32;
+    const uint8_t * const weights = (second ? a.packed_second : a.packed) + static_cast<int64_t>(expert) * a.bytes_per_expert;
+    const int rows_valid = max(1, min(32, a.out_features - n0));   // weight rows past the end repeat the last one (never stored)
+    const uint8_t * const rows = weights + static_cast<int64_t>(min(n0, a.out_features - 1)) * a.row_bytes;
+
+    // ---- the packed blocks: one super-block ahead in registers, the current one in the wave's LDS slot
+    constexpr int RAW_UNITS = K45 ? F::BLOCK_BYTES / 16 : 1;
+    constexpr int RAW_REGS = K45 ? (32 * RAW_UNITS + 63) / 64 : 1;
+    using W = WideStage<TYPE>;
+    constexpr int WIDE_REGS = WIDE ? W::template regs<32, 64>() : 1;
+    constexpr int SLOT_PITCH = K45 ? F::BLOCK_BYTES : (WIDE ? W::PITCH : F::RAW_PITCH);
+    constexpr int SLOT_FRONT = K45 ? 0 : (WIDE ? W::FRONT : F::RAW_SHIFT);
+    uint8_t * const slot = lds.raw[wave];
+    struct RawSet {
+        u32x4_t units[RAW_REGS];
+        WideRegs<WIDE_REGS> wide;
+    };
+    RawSet pending;
+    auto request = [&](int kb) __attribute__((always_inline)) {
+        kb = min(kb, super_blocks - 1);
+        if constexpr (K45) {
+            const uint8_t * base = rows + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
+#pragma unroll
+            for (int i = 0; i < RAW_REGS; ++i) {
+                const int id = min(lane + 64 * i, 32 * RAW_UNITS - 1);
+                const int row = id / RAW_UNITS;
+                const int unit = id - row * RAW_UNITS;
+                const uint32_t offset = __umul24(min(row, rows_valid - 1), static_cast<uint32_t>(a.row_bytes)) + unit * 16;
+                pending.units[i] = *reinterpret_cast<const u32x4_t *>(base + offset);
+            }
+        } else if constexpr (WIDE) {
+            wide_fetch<TYPE, 32, 64, WIDE_REGS>(pending.wide, rows, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
+        }
+    };
+    auto park = [&](int kb) __attribute__((always_inline)) {
+        kb = min(kb, super_blocks - 1);
+        // (the slot is written as words and read as bytes, halves and words: without these the compiler may move the
+        // writes across reads of another type; the hardware runs a wave's LDS accesses in order)
+        asm volatile("" ::: "memory");
+        if constexpr (K45) {
+#pragma unroll
+            for (int i = 0; i < RAW_REGS; ++i) {
+                const int id = min(lane + 64 * i, 32 * RAW_UNITS - 1);
+                *reinterpret_cast<u32x4_t *>(slot + id * 16) = pending.units[i];
+            }
+        } else if constexpr (WIDE) {
+            wide_park<TYPE, 32, 64, WIDE_REGS>(slot, pending.wide, rows, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
+        } else {
+            stage_blocks<TYPE>(slot, weights, a.row_bytes, min(n0, a.out_features - 1), a.out_features, kb, 32, lane, 64);
+        }
+        asm volatile("" ::: "memory");
+    };
+    request(0);
+
+    // ---- the weight normalisation: per weight row AND super-block here (2^s: the largest magnitude of the
+    // super-block's weights goes to [2^8, 2^9)), applied when a super-block's sum joins the row's: a scan of the row's
+    // scales ahead of the first block, as the kernel above does, would fetch a line of every block for four bytes of
+    // it, all waves at once, and the few waves of a short task have nothing to cover that with
+    auto block_power = [&](float reach, float & shrink) __attribute__((always_inline)) {
+        int exponent = static_cast<int>(__float_as_uint(reach) >> 23);   // biased
+        exponent = min(max(exponent, 9), 254);
+        if (half == 0) {
+            lds.column_power[wave][l32] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^s
+        }
+        shrink = __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-s
+    };
+
+    // ---- the activation rows (at most 32, from row_start: they may straddle two 32-row tiles of the workspace)
+    const int first_tile = row_start >> 5;
+    const uint8_t * const x_base = reinterpret_cast<const uint8_t *>(a.qx) + static_cast<int64_t>(first_tile) * blocks_per_row * 2048;
+    const uint8_t * const sums_base = reinterpret_cast<const uint8_t *>(a.block_sums) + static_cast<int64_t>(first_tile) * super_blocks * 512;
+    int lane_row = row_start + l32;
+    lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
+    const uint32_t x_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
+                            static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
+    const uint32_t sums_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
+                               static_cast<uint32_t>((lane_row & 31) * 16);
+    // Everything a super-block needs from memory is requested while the one before it is unpacked and multiplied, and
+    // awaited once, at its end: the packed blocks (this wave's), the wave's quarter of the task's activation fragments
+    // (which go to LDS for all four waves), the row's 2^(e - E) and block sums.  Loads return in order, so waiting
+    // for an activation fragment from the L2 in the middle of a super-block would also wait for the packed blocks
+    // behind which it was requested, and those come from HBM.
+    struct Incoming {
+        half8_t x[4];
+        float ratio;
+        uint4 sums;
+    };
+    Incoming incoming;
+    auto request_rows = [&](int kb) __attribute__((always_inline)) {
+        kb = min(kb, super_blocks - 1);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            incoming.x[i] = *reinterpret_cast<const half8_t *>(x_base + static_cast<int64_t>(kb * 16 + 4 * wave + i) * 1024 + x_lane);
+        }
+        incoming.ratio = a.power[static_cast<int64_t>(kb) * a.rows_padded + lane_row];
+        incoming.sums = make_uint4(0, 0, 0, 0);
+        if constexpr (K45) {
+            incoming.sums = *reinterpret_cast<const uint4 *>(sums_base + static_cast<int64_t>(kb) * 512 + sums_lane);
+        }
+    };
+    auto publish_rows = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            *reinterpret_cast<half8_t *>(&lds.x[(4 * wave + i) * 1024 + lane * 16]) = incoming.x[i];
+        }
+    };
+
+    const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    v16f acc = zero;     // of the super-block
+    v16f total = zero;   // of the row: sum over super-blocks of 2^s * acc
+    // The lane's 16 values of a block (k-half `half`: registers 0-3 hold its first eight, 4-7 the other eight) are the
+    // two fragments of reduction step 2 * block + half; the half-waves exchange what the other one multiplies, then
+    // `first` is step 2 * block and `other` step 2 * block + 1.
+    auto rescale = [&](half8_t fragment, half2_t ratio) __attribute__((always_inline)) {
+        const uint4 words = __builtin_bit_cast(uint4, fragment);
+        const uint4 scaled = make_uint4(half2_mul(words.x, ratio), half2_mul(words.y, ratio), half2_mul(words.z, ratio),
+                                        half2_mul(words.w, ratio));
+        return __builtin_bit_cast(half8_t, scaled);
+    };
+    // `step`: of the super-block (0..15); `fragments`: the super-block's activation fragments in LDS.  (Applying the
+    // row's 2^(e - E) to the super-block's sums instead of its fragments would save these multiplications; the
+    // compiler then schedules the fragment reads far ahead and spills what the wave has unpacked: measured slower.)
+    auto multiply_block = [&](uint32_t (&values)[8], int step, half2_t ratio, const uint8_t * fragments) __attribute__((always_inline)) {
+        uint32_t first[4], other[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const auto swapped = __builtin_amdgcn_permlane32_swap(values[i], values[4 + i], false, false);
+            first[i] = swapped[0];
+            other[i] = swapped[1];
+        }
+        const half8_t x0 = *reinterpret_cast<const half8_t *>(fragments + step * 1024 + lane * 16);
+        const half8_t x1 = *reinterpret_cast<const half8_t *>(fragments + (step + 1) * 1024 + lane * 16);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, make_uint4(first[0], first[1], first[2], first[3])),
+                                                     rescale(x0, ratio), acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, make_uint4(other[0], other[1], other[2], other[3])),
+                                                     rescale(x1, ratio), acc, 0, 0, 0);
+    };
+
+    const uint8_t * const blk = slot + l32 * SLOT_PITCH + SLOT_FRONT;
+    request_rows(0);
+    park(0);
+    publish_rows();
+    group_barrier();
+#pragma unroll 1
+    for (int kb = 0; kb < super_blocks; ++kb) {
+        const half2_t ratio = {static_cast<_Float16>(incoming.ratio), static_cast<_Float16>(incoming.ratio)};
+        const uint4 sums = incoming.sums;
+        const uint8_t * const fragments = lds.x;
+        request(kb + 1);
+        request_rows(kb + 1);
+        if constexpr (K45) {
+            constexpr int QS = TYPE == Q4_K ? 16 : 48;
+            const u32x4_t header = *reinterpret_cast<const u32x4_t *>(blk);
+            u32x4_t planes = {0, 0, 0, 0};
+            if constexpr (TYPE == Q5_K) {
+                planes = *reinterpret_cast<const u32x4_t *>(blk + 16 + 16 * half);
+            }
+            const uint32_t plane_word[4] = {planes.x, planes.y, planes.z, planes.w};
+            float shrink;
+            block_power(fmaxf(fabsf(half_bits_to_float(header.x & 0xffffu)) * weight_reach<TYPE>(),
+                              fabsf(half_bits_to_float(header.x >> 16)) * 63.0f), shrink);
+            const float d = half_bits_to_float(header.x & 0xffffu) * shrink;
+            auto chunk = [&](auto stage_tag, auto pair_tag) __attribute__((always_inline)) {
+                constexpr int S = decltype(stage_tag)::value;
+                constexpr int P = decltype(pair_tag)::value;
+                // (read where it is used: the other waves of the SIMD cover the LDS round trip, and the registers
+                // that an early read would hold are what keeps a stage of activation fragments in flight)
+                const u32x4_t nibbles = *reinterpret_cast<const u32x4_t *>(blk + QS + (2 * S + P) * 32 + 16 * half);
+                constexpr int G = 4 * S + 2 * P;   // low nibbles: group G, high nibbles: group G + 1
+                int sc_low, sc_high, unused;
+                k45_group_scale_min<G>(header.y, header.z, header.w, sc_low, unused);
+                k45_group_scale_min<G + 1>(header.y, header.z, header.w, sc_high, unused);
+                const HalfScale scale_low = half_scale_of(d * static_cast<float>(sc_low));
+                const HalfScale scale_high = half_scale_of(d * static_cast<float>(sc_high));
+                const uint32_t word[4] = {nibbles.x, nibbles.y, nibbles.z, nibbles.w};
+                uint32_t low[8], high[8];
+#pragma unroll
+                for (int w = 0; w < 4; ++w) {
+                    uint32_t bytes_low = word[w] & 0x0f0f0f0fu;
+                    uint32_t bytes_high = (word[w] >> 4) & 0x0f0f0f0fu;
+                    if constexpr (TYPE == Q5_K) {
+                        if constexpr (G <= 3) {
+                            bytes_low |= (plane_word[w] << (4 - G)) & 0x10101010u;
+                            bytes_high |= (plane_word[w] << (3 - G)) & 0x10101010u;
+                        } else {
+                            bytes_low |= (plane_word[w] >> (G - 4)) & 0x10101010u;
+                            bytes_high |= (plane_word[w] >> (G - 3)) & 0x10101010u;
+                        }
+                    }
+                    scaled_halves(bytes_low, scale_low, low[2 * w], low[2 * w + 1]);
+                    scaled_halves(bytes_high, scale_high, high[2 * w], high[2 * w + 1]);
+                }
+                multiply_block(low, 8 * S + 4 * P, ratio, fragments);
+                multiply_block(high, 8 * S + 4 * P + 2, ratio, fragments);
+            };
+            chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
+            chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
+            {   // the super-block's extra reduction step: block minima x block sums
+                int sc, mn[8];
+                k45_group_scale_min<0>(header.y, header.z, header.w, sc, mn[0]);
+                k45_group_scale_min<1>(header.y, header.z, header.w, sc, mn[1]);
+                k45_group_scale_min<2>(header.y, header.z, header.w, sc, mn[2]);
+                k45_group_scale_min<3>(header.y, header.z, header.w, sc, mn[3]);
+                k45_group_scale_min<4>(header.y, header.z, header.w, sc, mn[4]);
+                k45_group_scale_min<5>(header.y, header.z, header.w, sc, mn[5]);
+                k45_group_scale_min<6>(header.y, header.z, header.w, sc, mn[6]);
+                k45_group_scale_min<7>(header.y, header.z, header.w, sc, mn[7]);
+                const float minus = -half_bits_to_float(header.x >> 16) * shrink;
+                uint32_t packed[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const half2_t pair = {static_cast<_Float16>(minus * static_cast<float>(mn[2 * i])),
+                                          static_cast<_Float16>(minus * static_cast<float>(mn[2 * i + 1]))};
+                    packed[i] = half != 0 ? 0u : __builtin_bit_cast(uint32_t, pair);
+                }
+                const half8_t block_sums = rescale(__builtin_bit_cast(half8_t, half != 0 ? make_uint4(0, 0, 0, 0) : sums), ratio);
+                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
+                    __builtin_bit_cast(half8_t, make_uint4(packed[0], packed[1], packed[2], packed[3])), block_sums, acc, 0, 0, 0);
+            }
+            chunk(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
+            chunk(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
+        } else {
+            const auto * const grid = &lds.codebook;
+            float shrink;
+            block_power(fabsf(half_bits_to_float(lds_u16(blk + scale_offset<TYPE>()))) * weight_reach<TYPE>(), shrink);
+            const _Float16 h = static_cast<_Float16>(half_weight_scale<TYPE>(blk) * shrink);
+            const half2_t scale = {h, h};
+#pragma unroll
+            for (int b = 0; b < 8; ++b) {
+                uint32_t first[8], fine[8];
+                decode16_half<TYPE>(blk, 2 * b + half, grid, first, fine);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    if constexpr (TYPE == Q6_K) {
+                        first[i] = half2_fma(first[i], scale, __builtin_bit_cast(half2_t, half2_mul(fine[i], scale)));
+                    } else {
+                        first[i] = half2_mul(first[i], scale);
+                    }
+                }
+                multiply_block(first, 2 * b, ratio, fragments);
+            }
+        }
+        // (everything of this super-block has been read from the slot: the next one goes there; the next fragments
+        // replace this super-block's once every wave is done with them.  A second fragment buffer would save this
+        // barrier and cost the third workgroup per CU.)
+        park(kb + 1);
+        group_barrier();
+        publish_rows();
+        // the super-block's sums join the row's, each column with the power of two its weights were divided by
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float4 column_power = *reinterpret_cast<const float4 *>(&lds.column_power[wave][8 * j + 4 * half]);
+            total[4 * j + 0] = __builtin_fmaf(acc[4 * j + 0], column_power.x, total[4 * j + 0]);
+            total[4 * j + 1] = __builtin_fmaf(acc[4 * j + 1], column_power.y, total[4 * j + 1]);
+            total[4 * j + 2] = __builtin_fmaf(acc[4 * j + 2], column_power.z, total[4 * j + 2]);
+            total[4 * j + 3] = __builtin_fmaf(acc[4 * j + 3], column_power.w, total[4 * j + 3]);
+        }
+        acc = zero;
+        group_barrier();
+    }
+
+    // ---- epilogue: scale by 2^(E[r] + S[n]) and store 32 rows x 32 columns
+    {
+        const float row_power = a.row_power[lane_row];
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            acc[v] = total[v] * row_power;
+        }
+        uint16_t * const y = (second ? a.y_second : a.y) + static_cast<int64_t>(row_start) * a.out_features + n0;
+        const bool wide_rows = (a.out_features & 7) == 0;
+        uint16_t * const row = y + l32 * static_cast<int64_t>(a.out_features);
+        const int valid_rows = row_end - row_start;
+        const int valid_cols = a.out_features - n0;
+#pragma unroll
+        for (int m = 0; m < 2; ++m) {
+            const uint32_t p0 = pack_bf16x2(acc[8 * m + 0], acc[8 * m + 1]);
+            const uint32_t p1 = pack_bf16x2(acc[8 * m + 2], acc[8 * m + 3]);
+            const uint32_t q0 = pack_bf16x2(acc[8 * m + 4], acc[8 * m + 5]);
+            const uint32_t q1 = pack_bf16x2(acc[8 * m + 6], acc[8 * m + 7]);
+            const auto s0 = __builtin_amdgcn_permlane32_swap(p0, q0, false, false);
+            const auto s1 = __builtin_amdgcn_permlane32_swap(p1, q1, false, false);
+            const uint32_t words[4] = {s0[0], s1[0], s0[1], s1[1]};
+            const int c = 16 * m + 8 * half;
+            if (l32 < valid_rows && c < valid_cols) {
+                if (wide_rows && c + 8 <= valid_cols) {
+                    *reinterpret_cast<uint4 *>(row + c) = make_uint4(words[0], words[1], words[2], words[3]);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) {
+                        if (c + e < valid_cols) {
+                            row[c + e] = static_cast<uint16_t>(words[e >> 1] >> (16 * (e & 1)));
+                        }
+                    }
+                }
+            }
+        }
+    }
+    group_barrier();   // (the next item reuses the LDS buffers)
+    }
+}
+
+
+template <int TYPE, bool WIDE>
+__global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(const ForwardArgs a, const int total_slots,
+                                                                            const int main_blocks) {
     using F = Format<TYPE>;
     using L = ScaledLds<TYPE>;
     constexpr bool K45 = L::K45;
-    __shared__ L lds;
+    constexpr int SHORT_GROUPS = FSC_THREADS / (64 * FSS_WAVES);
+    union Shared {
+        L role_split;
+        ShortLds<TYPE> short_groups[SHORT_GROUPS];
+    };
+    __shared__ Shared shared;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -174,11 +583,22 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     const int l32 = lane & 31;
     const int half = lane >> 5;
 
-    // item table: slot i of this workgroup is position blockIdx.x + i * gridDim.x of the launch order (gridDim.x is
+    // The workgroups behind the role-split ones run the groups of at most 32 rows.  Workgroups start in the order of
+    // their numbers and one fills a CU, so these start on the CUs whose role-split workgroup has run out of items while
+    // the last round of items still occupies the others.
+    if (static_cast<int>(blockIdx.x) >= main_blocks) {
+        const int group = __builtin_amdgcn_readfirstlane(tid / (64 * FSS_WAVES));
+        short_group_items<TYPE, WIDE>(a, shared.short_groups[group], tid % (64 * FSS_WAVES), group,
+                                      static_cast<int>(gridDim.x) - main_blocks);
+        return;
+    }
+    L & lds = shared.role_split;
+
+    // item table: slot i of this workgroup is position blockIdx.x + i * main_blocks of the launch order (main_blocks is
     // a multiple of the XCD count, so all of them map to this workgroup's XCD); empty slots are squeezed out
     if (wave == 0) {
         ScaledItem item = {0, 0, 0, -1};
-        const int64_t linear = blockIdx.x + static_cast<int64_t>(lane) * gridDim.x;
+        const int64_t linear = blockIdx.x + static_cast<int64_t>(lane) * main_blocks;
         if (linear < total_slots) {
             int n_tile, expert, row_start, row_end;
             bool second;
@@ -782,379 +1202,23 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     }
 }
 
-// ---- groups of at most 32 rows ---------------------------------------------------------------------------------
-// A task of a few rows costs the kernel above what a full one costs its unpacking waves, while seven of its eight
-// multiplying waves have nothing to do: on a routing with many small groups a third of its time went into 1.5 % of the
-// rows.  Such tasks (the list keeps whole groups of at most 32 rows behind the others) go to this kernel instead, in
-// which every wave unpacks: a wave owns 32 weight rows of the task's column tile and the task's one 32-row activation
-// tile, from the packed blocks to the stored results, and never meets another wave.  Its fp16 weights stay in
-// registers: the lane that unpacks k-half h of a 32-value block of weight row n holds exactly the two matrix-instruction
-// fragments of reduction step 2 * block + h, and one exchange between the half-waves (v_permlane32_swap) per register
-// puts them where the instruction wants them.  Three such workgroups of four waves share a CU, so that twelve waves keep
-// the vector pipe busy where four did.  The algebra is that of the kernel above except for the weight normalisation,
-// which is per super-block here (see below): the two kernels agree to fp32 rounding of that last step, not bit for bit.
-constexpr int FSS_WAVES = 4;
-
-template <int TYPE>
-struct ShortLds {
-    static constexpr int RAW_SLOT = ScaledLds<TYPE>::RAW_SLOT;
-    alignas(16) uint8_t raw[FSS_WAVES][32 * RAW_SLOT];   // per wave: the packed blocks of one super-block
-    alignas(16) uint8_t x[16 * 1024];                    // the task's activation fragments of one super-block
-    alignas(16) float column_power[FSS_WAVES][32];       // 2^s of the wave's weight rows in the current super-block
-    std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;
-};
-
-template <int TYPE, bool WIDE>
-__global__ __launch_bounds__(64 * FSS_WAVES, 3) void mmq_forward_scaled_short_kernel(const ForwardArgs a) {
-    using F = Format<TYPE>;
-    using L = ShortLds<TYPE>;
-    constexpr bool K45 = TYPE == Q4_K || TYPE == Q5_K;
-    __shared__ L lds;
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int l32 = lane & 31;
-    const int half = lane >> 5;
-    if constexpr (TYPE == IQ2_S) {
-        expand_iq2s_selectors(lds.codebook, tid, 64 * FSS_WAVES);
-        __syncthreads();
-    }
-    // The number of short tasks is known on the device only (one round trip to read it): a fixed number of workgroups,
-    // three per CU, take the (short task, column tile and projection) items in turn.
-    const int inner = a.n_tiles * a.projections;
-    const int tasks = a.task_count[0];
-    const int first_short = min(a.task_early[0], tasks);
-    const int items = (tasks - first_short) * inner;
-#pragma unroll 1
-    for (int item = blockIdx.x; item < items; item += gridDim.x) {
-    const int task = first_short + item / inner;
-    int tile = item % inner;
-    const bool second = tile >= a.n_tiles;
-    tile -= second ? a.n_tiles : 0;
-    // (a wave whose weight rows lie past the end of the matrix repeats the last row and stores nothing: the
-    // workgroup's barriers need it)
-    const int n0 = tile * FWD_TN + 32 * wave;
-    const int expert = a.task_expert[task];
-    const int row_start = a.task_row_start[task];
-    const int row_end = a.task_row_end[task];
-    const int super_blocks = a.in_features / QK_K;
-    const int blocks_per_row = a.in_features / 32;
-    const uint8_t * const weights = (second ? a.packed_second : a.packed) + static_cast<int64_t>(expert) * a.bytes_per_expert;
-    const int rows_valid = max(1, min(32, a.out_features - n0));   // weight rows past the end repeat the last one (never stored)
-    const uint8_t * const rows = weights + static_cast<int64_t>(min(n0, a.out_features - 1)) * a.row_bytes;
-
-    // ---- the packed blocks: one super-block ahead in registers, the current one in the wave's LDS slot
-    constexpr int RAW_UNITS = K45 ? F::BLOCK_BYTES / 16 : 1;
-    constexpr int RAW_REGS = K45 ? (32 * RAW_UNITS + 63) / 64 : 1;
-    using W = WideStage<TYPE>;
-    constexpr int WIDE_REGS = WIDE ? W::template regs<32, 64>() : 1;
-    constexpr int SLOT_PITCH = K45 ? F::BLOCK_BYTES : (WIDE ? W::PITCH : F::RAW_PITCH);
-    constexpr int SLOT_FRONT = K45 ? 0 : (WIDE ? W::FRONT : F::RAW_SHIFT);
-    uint8_t * const slot = lds.raw[wave];
-    struct RawSet {
-        u32x4_t units[RAW_REGS];
-        WideRegs<WIDE_REGS> wide;
-    };
-    RawSet pending;
-    auto request = [&](int kb) __attribute__((always_inline)) {
-        kb = min(kb, super_blocks - 1);
-        if constexpr (K45) {
-            const uint8_t * base = rows + static_cast<int64_t>(kb) * F::BLOCK_BYTES;
-#pragma unroll
-            for (int i = 0; i < RAW_REGS; ++i) {
-                const int id = min(lane + 64 * i, 32 * RAW_UNITS - 1);
-                const int row = id / RAW_UNITS;
-                const int unit = id - row * RAW_UNITS;
-                const uint32_t offset = __umul24(min(row, rows_valid - 1), static_cast<uint32_t>(a.row_bytes)) + unit * 16;
-                pending.units[i] = *reinterpret_cast<const u32x4_t *>(base + offset);
-            }
-        } else if constexpr (WIDE) {
-            wide_fetch<TYPE, 32, 64, WIDE_REGS>(pending.wide, rows, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
-        }
-    };
-    auto park = [&](int kb) __attribute__((always_inline)) {
-        kb = min(kb, super_blocks - 1);
-        // (the slot is written as words and read as bytes, halves and words: without these the compiler may move the
-        // writes across reads of another type; the hardware runs a wave's LDS accesses in order)
-        asm volatile("" ::: "memory");
-        if constexpr (K45) {
-#pragma unroll
-            for (int i = 0; i < RAW_REGS; ++i) {
-                const int id = min(lane + 64 * i, 32 * RAW_UNITS - 1);
-                *reinterpret_cast<u32x4_t *>(slot + id * 16) = pending.units[i];
-            }
-        } else if constexpr (WIDE) {
-            wide_park<TYPE, 32, 64, WIDE_REGS>(slot, pending.wide, rows, static_cast<int>(a.row_bytes), rows_valid, kb, lane);
-        } else {
-            stage_blocks<TYPE>(slot, weights, a.row_bytes, min(n0, a.out_features - 1), a.out_features, kb, 32, lane, 64);
-        }
-        asm volatile("" ::: "memory");
-    };
-    request(0);
-
-    // ---- the weight normalisation: per weight row AND super-block here (2^s: the largest magnitude of the
-    // super-block's weights goes to [2^8, 2^9)), applied when a super-block's sum joins the row's: a scan of the row's
-    // scales ahead of the first block, as the kernel above does, would fetch a line of every block for four bytes of
-    // it, all waves at once, and the few waves of a short task have nothing to cover that with
-    auto block_power = [&](float reach, float & shrink) __attribute__((always_inline)) {
-        int exponent = static_cast<int>(__float_as_uint(reach) >> 23);   // biased
-        exponent = min(max(exponent, 9), 254);
-        if (half == 0) {
-            lds.column_power[wave][l32] = __uint_as_float(static_cast<uint32_t>(exponent - 8) << 23);   // 2^s
-        }
-        shrink = __uint_as_float(static_cast<uint32_t>(262 - exponent) << 23);   // 2^-s
-    };
-
-    // ---- the activation rows (at most 32, from row_start: they may straddle two 32-row tiles of the workspace)
-    const int first_tile = row_start >> 5;
-    const uint8_t * const x_base = reinterpret_cast<const uint8_t *>(a.qx) + static_cast<int64_t>(first_tile) * blocks_per_row * 2048;
-    const uint8_t * const sums_base = reinterpret_cast<const uint8_t *>(a.block_sums) + static_cast<int64_t>(first_tile) * super_blocks * 512;
-    int lane_row = row_start + l32;
-    lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
-    const uint32_t x_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
-                            static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
-    const uint32_t sums_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
-                               static_cast<uint32_t>((lane_row & 31) * 16);
-    // Everything a super-block needs from memory is requested while the one before it is unpacked and multiplied, and
-    // awaited once, at its end: the packed blocks (this wave's), the wave's quarter of the task's activation fragments
-    // (which go to LDS for all four waves), the row's 2^(e - E) and block sums.  Loads return in order, so waiting
-    // for an activation fragment from the L2 in the middle of a super-block would also wait for the packed blocks
-    // behind which it was requested, and those come from HBM.
-    struct Incoming {
-        half8_t x[4];
-        float ratio;
-        uint4 sums;
-    };
-    Incoming incoming;
-    auto request_rows = [&](int kb) __attribute__((always_inline)) {
-        kb = min(kb, super_blocks - 1);
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            incoming.x[i] = *reinterpret_cast<const half8_t *>(x_base + static_cast<int64_t>(kb * 16 + 4 * wave + i) * 1024 + x_lane);
-        }
-        incoming.ratio = a.power[static_cast<int64_t>(kb) * a.rows_padded + lane_row];
-        incoming.sums = make_uint4(0, 0, 0, 0);
-        if constexpr (K45) {
-            incoming.sums = *reinterpret_cast<const uint4 *>(sums_base + static_cast<int64_t>(kb) * 512 + sums_lane);
-        }
-    };
-    auto publish_rows = [&]() __attribute__((always_inline)) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            *reinterpret_cast<half8_t *>(&lds.x[(4 * wave + i) * 1024 + lane * 16]) = incoming.x[i];
-        }
-    };
-
-    const v16f zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    v16f acc = zero;     // of the super-block
-    v16f total = zero;   // of the row: sum over super-blocks of 2^s * acc
-    // The lane's 16 values of a block (k-half `half`: registers 0-3 hold its first eight, 4-7 the other eight) are the
-    // two fragments of reduction step 2 * block + half; the half-waves exchange what the other one multiplies, then
-    // `first` is step 2 * block and `other` step 2 * block + 1.
-    auto rescale = [&](half8_t fragment, half2_t ratio) __attribute__((always_inline)) {
-        const uint4 words = __builtin_bit_cast(uint4, fragment);
-        const uint4 scaled = make_uint4(half2_mul(words.x, ratio), half2_mul(words.y, ratio), half2_mul(words.z, ratio),
-                                        half2_mul(words.w, ratio));
-        return __builtin_bit_cast(half8_t, scaled);
-    };
-    // `step`: of the super-block (0..15); `fragments`: the super-block's activation fragments in LDS.  (Applying the
-    // row's 2^(e - E) to the super-block's sums instead of its fragments would save these multiplications; the
-    // compiler then schedules the fragment reads far ahead and spills what the wave has unpacked: measured slower.)
-    auto multiply_block = [&](uint32_t (&values)[8], int step, half2_t ratio, const uint8_t * fragments) __attribute__((always_inline)) {
-        uint32_t first[4], other[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            const auto swapped = __builtin_amdgcn_permlane32_swap(values[i], values[4 + i], false, false);
-            first[i] = swapped[0];
-            other[i] = swapped[1];
-        }
-        const half8_t x0 = *reinterpret_cast<const half8_t *>(fragments + step * 1024 + lane * 16);
-        const half8_t x1 = *reinterpret_cast<const half8_t *>(fragments + (step + 1) * 1024 + lane * 16);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, make_uint4(first[0], first[1], first[2], first[3])),
-                                                     rescale(x0, ratio), acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(half8_t, make_uint4(other[0], other[1], other[2], other[3])),
-                                                     rescale(x1, ratio), acc, 0, 0, 0);
-    };
-
-    const uint8_t * const blk = slot + l32 * SLOT_PITCH + SLOT_FRONT;
-    request_rows(0);
-    park(0);
-    publish_rows();
-    __syncthreads();
-#pragma unroll 1
-    for (int kb = 0; kb < super_blocks; ++kb) {
-        const half2_t ratio = {static_cast<_Float16>(incoming.ratio), static_cast<_Float16>(incoming.ratio)};
-        const uint4 sums = incoming.sums;
-        const uint8_t * const fragments = lds.x;
-        request(kb + 1);
-        request_rows(kb + 1);
-        if constexpr (K45) {
-            constexpr int QS = TYPE == Q4_K ? 16 : 48;
-            const u32x4_t header = *reinterpret_cast<const u32x4_t *>(blk);
-            u32x4_t planes = {0, 0, 0, 0};
-            if constexpr (TYPE == Q5_K) {
-                planes = *reinterpret_cast<const u32x4_t *>(blk + 16 + 16 * half);
-            }
-            const uint32_t plane_word[4] = {planes.x, planes.y, planes.z, planes.w};
-            float shrink;
-            block_power(fmaxf(fabsf(half_bits_to_float(header.x & 0xffffu)) * weight_reach<TYPE>(),
-                              fabsf(half_bits_to_float(header.x >> 16)) * 63.0f), shrink);
-            const float d = half_bits_to_float(header.x & 0xffffu) * shrink;
-            auto chunk = [&](auto stage_tag, auto pair_tag) __attribute__((always_inline)) {
-                constexpr int S = decltype(stage_tag)::value;
-                constexpr int P = decltype(pair_tag)::value;
-                // (read where it is used: the other waves of the SIMD cover the LDS round trip, and the registers
-                // that an early read would hold are what keeps a stage of activation fragments in flight)
-                const u32x4_t nibbles = *reinterpret_cast<const u32x4_t *>(blk + QS + (2 * S + P) * 32 + 16 * half);
-                constexpr int G = 4 * S + 2 * P;   // low nibbles: group G, high nibbles: group G + 1
-                int sc_low, sc_high, unused;
-                k45_group_scale_min<G>(header.y, header.z, header.w, sc_low, unused);
-                k45_group_scale_min<G + 1>(header.y, header.z, header.w, sc_high, unused);
-                const HalfScale scale_low = half_scale_of(d * static_cast<float>(sc_low));
-                const HalfScale scale_high = half_scale_of(d * static_cast<float>(sc_high));
-                const uint32_t word[4] = {nibbles.x, nibbles.y, nibbles.z, nibbles.w};
-                uint32_t low[8], high[8];
-#pragma unroll
-                for (int w = 0; w < 4; ++w) {
-                    uint32_t bytes_low = word[w] & 0x0f0f0f0fu;
-                    uint32_t bytes_high = (word[w] >> 4) & 0x0f0f0f0fu;
-                    if constexpr (TYPE == Q5_K) {
-                        if constexpr (G <= 3) {
-                            bytes_low |= (plane_word[w] << (4 - G)) & 0x10101010u;
-                            bytes_high |= (plane_word[w] << (3 - G)) & 0x10101010u;
-                        } else {
-                            bytes_low |= (plane_word[w] >> (G - 4)) & 0x10101010u;
-                            bytes_high |= (plane_word[w] >> (G - 3)) & 0x10101010u;
-                        }
-                    }
-                    scaled_halves(bytes_low, scale_low, low[2 * w], low[2 * w + 1]);
-                    scaled_halves(bytes_high, scale_high, high[2 * w], high[2 * w + 1]);
-                }
-                multiply_block(low, 8 * S + 4 * P, ratio, fragments);
-                multiply_block(high, 8 * S + 4 * P + 2, ratio, fragments);
-            };
-            chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 0>{});
-            chunk(std::integral_constant<int, 0>{}, std::integral_constant<int, 1>{});
-            {   // the super-block's extra reduction step: block minima x block sums
-                int sc, mn[8];
-                k45_group_scale_min<0>(header.y, header.z, header.w, sc, mn[0]);
-                k45_group_scale_min<1>(header.y, header.z, header.w, sc, mn[1]);
-                k45_group_scale_min<2>(header.y, header.z, header.w, sc, mn[2]);
-                k45_group_scale_min<3>(header.y, header.z, header.w, sc, mn[3]);
-                k45_group_scale_min<4>(header.y, header.z, header.w, sc, mn[4]);
-                k45_group_scale_min<5>(header.y, header.z, header.w, sc, mn[5]);
-                k45_group_scale_min<6>(header.y, header.z, header.w, sc, mn[6]);
-                k45_group_scale_min<7>(header.y, header.z, header.w, sc, mn[7]);
-                const float minus = -half_bits_to_float(header.x >> 16) * shrink;
-                uint32_t packed[4];
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    const half2_t pair = {static_cast<_Float16>(minus * static_cast<float>(mn[2 * i])),
-                                          static_cast<_Float16>(minus * static_cast<float>(mn[2 * i + 1]))};
-                    packed[i] = half != 0 ? 0u : __builtin_bit_cast(uint32_t, pair);
-                }
-                const half8_t block_sums = rescale(__builtin_bit_cast(half8_t, half != 0 ? make_uint4(0, 0, 0, 0) : sums), ratio);
-                acc = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                    __builtin_bit_cast(half8_t, make_uint4(packed[0], packed[1], packed[2], packed[3])), block_sums, acc, 0, 0, 0);
-            }
-            chunk(std::integral_constant<int, 1>{}, std::integral_constant<int, 0>{});
-            chunk(std::integral_constant<int, 1>{}, std::integral_constant<int, 1>{});
-        } else {
-            const auto * const grid = &lds.codebook;
-            float shrink;
-            block_power(fabsf(half_bits_to_float(lds_u16(blk + scale_offset<TYPE>()))) * weight_reach<TYPE>(), shrink);
-            const _Float16 h = static_cast<_Float16>(half_weight_scale<TYPE>(blk) * shrink);
-            const half2_t scale = {h, h};
-#pragma unroll
-            for (int b = 0; b < 8; ++b) {
-                uint32_t first[8], fine[8];
-                decode16_half<TYPE>(blk, 2 * b + half, grid, first, fine);
-#pragma unroll
-                for (int i = 0; i < 8; ++i) {
-                    if constexpr (TYPE == Q6_K) {
-                        first[i] = half2_fma(first[i], scale, __builtin_bit_cast(half2_t, half2_mul(fine[i], scale)));
-                    } else {
-                        first[i] = half2_mul(first[i], scale);
-                    }
-                }
-                multiply_block(first, 2 * b, ratio, fragments);
-            }
-        }
-        // (everything of this super-block has been read from the slot: the next one goes there; the next fragments
-        // replace this super-block's once every wave is done with them.  A second fragment buffer would save this
-        // barrier and cost the third workgroup per CU.)
-        park(kb + 1);
-        __syncthreads();
-        publish_rows();
-        // the super-block's sums join the row's, each column with the power of two its weights were divided by
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const float4 column_power = *reinterpret_cast<const float4 *>(&lds.column_power[wave][8 * j + 4 * half]);
-            total[4 * j + 0] = __builtin_fmaf(acc[4 * j + 0], column_power.x, total[4 * j + 0]);
-            total[4 * j + 1] = __builtin_fmaf(acc[4 * j + 1], column_power.y, total[4 * j + 1]);
-            total[4 * j + 2] = __builtin_fmaf(acc[4 * j + 2], column_power.z, total[4 * j + 2]);
-            total[4 * j + 3] = __builtin_fmaf(acc[4 * j + 3], column_power.w, total[4 * j + 3]);
-        }
-        acc = zero;
-        __syncthreads();
-    }
-
-    // ---- epilogue: scale by 2^(E[r] + S[n]) and store 32 rows x 32 columns
-    {
-        const float row_power = a.row_power[lane_row];
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            acc[v] = total[v] * row_power;
-        }
-        uint16_t * const y = (second ? a.y_second : a.y) + static_cast<int64_t>(row_start) * a.out_features + n0;
-        const bool wide_rows = (a.out_features & 7) == 0;
-        uint16_t * const row = y + l32 * static_cast<int64_t>(a.out_features);
-        const int valid_rows = row_end - row_start;
-        const int valid_cols = a.out_features - n0;
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            const uint32_t p0 = pack_bf16x2(acc[8 * m + 0], acc[8 * m + 1]);
-            const uint32_t p1 = pack_bf16x2(acc[8 * m + 2], acc[8 * m + 3]);
-            const uint32_t q0 = pack_bf16x2(acc[8 * m + 4], acc[8 * m + 5]);
-            const uint32_t q1 = pack_bf16x2(acc[8 * m + 6], acc[8 * m + 7]);
-            const auto s0 = __builtin_amdgcn_permlane32_swap(p0, q0, false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(p1, q1, false, false);
-            const uint32_t words[4] = {s0[0], s1[0], s0[1], s1[1]};
-            const int c = 16 * m + 8 * half;
-            if (l32 < valid_rows && c < valid_cols) {
-                if (wide_rows && c + 8 <= valid_cols) {
-                    *reinterpret_cast<uint4 *>(row + c) = make_uint4(words[0], words[1], words[2], words[3]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        if (c + e < valid_cols) {
-                            row[c + e] = static_cast<uint16_t>(words[e >> 1] >> (16 * (e & 1)));
-                        }
-                    }
-                }
-            }
-        }
-    }
-    __syncthreads();   // (the next item reuses the LDS buffers)
-    }
-}
-
-
 template <int TYPE>
 static hipError_t launch_forward_scaled_typed(const ForwardArgs & call, hipStream_t stream) {
     ForwardArgs args = call;
     const int64_t total = static_cast<int64_t>(args.n_tiles) * args.projections *
                           (args.task_count != nullptr ? xcd_chunk_slots(args.task_slots) : pad_task_slots(args.task_slots, FWD_XCD_RUN));
-    // grouped calls: whole groups of at most 32 rows are listed behind the other tasks and take the kernel whose
-    // waves all unpack (three workgroups per CU share its items; fewer when there cannot be that many)
+    // grouped calls: whole groups of at most 32 rows are listed behind the other tasks and go to workgroups of their own,
+    // each of which runs up to three such items at a time (one per CU suffices: they take their items in rounds)
+    constexpr int SHORT_GROUPS = FSC_THREADS / (64 * FSS_WAVES);
     const int64_t short_items = args.task_count != nullptr ? static_cast<int64_t>(args.task_slots) * args.n_tiles * args.projections : 0;
-    const int64_t short_grid = short_items < 3 * FSC_GRID ? short_items : 3 * FSC_GRID;
-    if (total <= 0 || total > 0x7fffffffLL || short_grid > 0x7fffffffLL || args.swiglu != 0 || args.in_features > (1 << 22)) {
+    const int64_t short_units = (short_items + SHORT_GROUPS - 1) / SHORT_GROUPS;
+    const int64_t short_blocks = short_units < FSC_GRID ? short_units : FSC_GRID;
+    if (total <= 0 || total > 0x7fffffffLL || args.swiglu != 0 || args.in_features > (1 << 22)) {
         return hipErrorInvalidValue;
     }
     args.early_only = args.task_count != nullptr ? 1 : 0;
-    // one workgroup per CU; more when a workgroup's table would not hold its share (a multiple of the XCD count
-    // either way, so that a workgroup's items stay on its XCD)
+    // one role-split workgroup per CU; more when a workgroup's table would not hold its share (a multiple of the XCD
+    // count either way, so that a workgroup's items stay on its XCD)
     int64_t grid = FSC_GRID;
     if (total > grid * FSC_MAX_ITEMS) {
         grid = ((total + FSC_MAX_ITEMS - 1) / FSC_MAX_ITEMS + XCDS - 1) / XCDS * XCDS;
@@ -1167,23 +1231,13 @@ static hipError_t launch_forward_scaled_typed(const ForwardArgs & call, hipStrea
     if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
         wide = args.wide != 0;
     }
+    const unsigned blocks = static_cast<unsigned>(grid + short_blocks);
     if (wide) {
         if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
-            mmq_forward_scaled_kernel<TYPE, true><<<static_cast<unsigned>(grid), FSC_THREADS, 0, stream>>>(args, static_cast<int>(total));
+            mmq_forward_scaled_kernel<TYPE, true><<<blocks, FSC_THREADS, 0, stream>>>(args, static_cast<int>(total), static_cast<int>(grid));
         }
     } else {
-        mmq_forward_scaled_kernel<TYPE, false><<<static_cast<unsigned>(grid), FSC_THREADS, 0, stream>>>(args, static_cast<int>(total));
-    }
-    hipError_t status = hipGetLastError();
-    if (status != hipSuccess || short_grid == 0) {
-        return status;
-    }
-    if (wide) {
-        if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
-            mmq_forward_scaled_short_kernel<TYPE, true><<<static_cast<unsigned>(short_grid), 64 * FSS_WAVES, 0, stream>>>(args);
-        }
-    } else {
-        mmq_forward_scaled_short_kernel<TYPE, false><<<static_cast<unsigned>(short_grid), 64 * FSS_WAVES, 0, stream>>>(args);
+        mmq_forward_scaled_kernel<TYPE, false><<<blocks, FSC_THREADS, 0, stream>>>(args, static_cast<int>(total), static_cast<int>(grid));
     }
     return hipGetLastError();
 }

@@ -157,14 +157,16 @@ static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t i
     return view;
 }
 
-// Tile tasks of the grouped operators: [count][early][expert x max][row_start x max][row_end x max].
+// Tile tasks of the grouped operators: [count][early][expert x max][row_start x max][row_end x max][cursor].
 // `early` is the number of tasks listed before the short ones (TaskBuild::late_rows); count when nothing is short.
+// `cursor` is zero when the list is built: a kernel whose workgroups take items of the list in turn counts them there.
 struct TaskList {
     int32_t * count;
     int32_t * early;
     int32_t * expert;
     int32_t * row_start;
     int32_t * row_end;
+    int32_t * cursor;
     int max_tasks;
 };
 
@@ -174,7 +176,7 @@ static inline int max_tasks_for(int64_t rows, int64_t groups, int row_tile) {
 
 static inline int64_t task_workspace_bytes(int64_t rows, int64_t groups) {
     // sized for the smallest tile any kernel uses so one buffer fits every path
-    return (2 + 3 * static_cast<int64_t>(max_tasks_for(rows, groups, GEMV_ROW_TILE))) *
+    return (3 + 3 * static_cast<int64_t>(max_tasks_for(rows, groups, GEMV_ROW_TILE))) *
            static_cast<int64_t>(sizeof(int32_t));
 }
 
@@ -186,6 +188,7 @@ static inline TaskList task_list_view(void * base, int64_t rows, int64_t groups,
     list.expert = list.count + 2;
     list.row_start = list.expert + list.max_tasks;
     list.row_end = list.row_start + list.max_tasks;
+    list.cursor = list.row_end + list.max_tasks;
     return list;
 }
 

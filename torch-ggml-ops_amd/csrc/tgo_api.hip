@@ -190,7 +190,7 @@ ProfileScope::~ProfileScope() {
 
 extern "C" {
 
-int tgo_version(void) { return 110; }
+int tgo_version(void) { return 111; }
 
 int tgo_profile_enable(int enabled) {
     std::lock_guard<std::mutex> lock(g_profile_mutex);

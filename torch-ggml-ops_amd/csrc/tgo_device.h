@@ -220,7 +220,9 @@ TGO_DEVICE void build_tasks(const TaskBuild & b, int tid) {
     if (tid == 0) {
         b.tasks.count[0] = min(running + running_late, b.tasks.max_tasks);
         b.tasks.early[0] = min(running, b.tasks.max_tasks);
-        b.tasks.cursor[0] = 0;
+    }
+    if (tid < TASK_CURSORS) {
+        b.tasks.cursor[tid * TASK_CURSOR_STRIDE] = 0;
     }
 }
 

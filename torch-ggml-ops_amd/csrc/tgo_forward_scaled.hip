@@ -185,7 +185,7 @@ struct ShortLds {
     alignas(16) uint8_t x[16 * 1024];                    // the task's activation fragments of one super-block
     alignas(16) float column_power[FSS_WAVES][32];       // 2^s of the wave's weight rows in the current super-block
     alignas(16) int arrived[FSS_WAVES];                  // barriers of the group that each of its waves has reached
-    int next_item;                                       // the item that the group has taken from the list
+    int next_item;                                       // the chunk of items that the group has taken from the list
     std::conditional_t<TYPE == IQ2_S, Iq2sSelectors, uint2> codebook;
 };
 
@@ -198,7 +198,10 @@ struct ShortLds {
 // take more than twice as long as one that is alone there, so towards the end of the list the later groups stop
 // taking items and the last ones are spread over the CUs.  Workgroups that start late, on the CUs of the role-split
 // workgroups that ran longest, simply take fewer.
-template <int TYPE, bool WIDE>
+// Without TRAILING the routine is a workgroup's whole program (one group: the workgroup's barrier serves) and the items
+// go round the `blocks` workgroups of a launch of its own: for rows of fewer than four super-blocks, whose items are too
+// short to pay for an item taken from a cursor (two dependent round trips to memory each).
+template <int TYPE, bool WIDE, bool TRAILING>
 TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, const int tid, const int group, const int blocks) {
     using F = Format<TYPE>;
     constexpr bool K45 = TYPE == Q4_K || TYPE == Q5_K;
@@ -218,6 +221,10 @@ TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, c
     int barriers_passed = 0;
     auto group_barrier = [&]() __attribute__((always_inline)) {
         ++barriers_passed;
+        if constexpr (!TRAILING) {
+            __syncthreads();
+            return;
+        }
         asm volatile("" ::: "memory");   // (the data accesses stay before the count)
         if (lane == 0) {
             *(volatile __attribute__((address_space(3))) int *)&lds.arrived[wave] = barriers_passed;
@@ -236,20 +243,49 @@ TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, c
     const int tasks = a.task_count[0];
     const int first_short = min(a.task_early[0], tasks);
     const int items = (tasks - first_short) * inner;
+    // Items are taken in chunks of at least four super-blocks of work, from TASK_CURSORS lists: chunk j belongs to list
+    // j % TASK_CURSORS, whose cursor counts the chunks taken from it.  (Atomic operations on one address complete one
+    // after the other, at some tens of nanoseconds each: a thousand items through one cursor cost more than they saved.)
+    // A group starts with the list of its workgroup's number and goes on to the others when that is used up.
+    const int chunk_items = max(1, 4 / (a.in_features / QK_K));
+    const int chunks = (items + chunk_items - 1) / chunk_items;
+    const int home = static_cast<int>(blockIdx.x) % TASK_CURSORS;
+    const int blocks_per_list = max(1, blocks / TASK_CURSORS);
+    int item = TRAILING ? 0 : static_cast<int>(blockIdx.x) - blocks + 1, item_end = 0;
 #pragma unroll 1
     for (;;) {
-    if (tid == 0) {
-        // (an estimate of what is left decides whether this group still takes part; the count itself is exact)
-        const int left = items - __hip_atomic_load(a.task_cursor, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        // (a group's first item: while any is left -- the groups that started with it are all busy as long; later: only
-        // if the groups before it, one more item each, would not finish the list)
-        const int taken = left > (barriers_passed == 0 ? 0 : group * blocks) ? atomicAdd(a.task_cursor, 1) : items;
-        *(volatile __attribute__((address_space(3))) int *)&lds.next_item = taken;
-    }
-    group_barrier();
-    const int item = __builtin_amdgcn_readfirstlane(*(const volatile __attribute__((address_space(3))) int *)&lds.next_item);
-    if (item >= items) {
-        break;
+    if constexpr (!TRAILING) {
+        item += blocks - 1;   // (with the increment at the end of an item: every blocks-th item, from the workgroup's number)
+        if (item >= items) {
+            break;
+        }
+    } else if (item == item_end) {
+        if (tid == 0) {
+            int chunk = -1;
+            for (int k = 0; k < TASK_CURSORS && chunk < 0; ++k) {
+                const int list = (home + k) % TASK_CURSORS;
+                int32_t * const cursor = a.task_cursor + list * TASK_CURSOR_STRIDE;
+                const int in_list = (chunks - list + TASK_CURSORS - 1) / TASK_CURSORS;   // chunks j = list (mod TASK_CURSORS)
+                // (an estimate of what is left decides whether this group still takes part; the count itself is exact)
+                const int left = in_list - __hip_atomic_load(cursor, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                // (a group's first chunk: while any is left -- the groups that started with it are all busy as long;
+                // later: only if the groups before it, one more chunk each, would not finish the list)
+                if (left > (barriers_passed == 0 ? 0 : group * blocks_per_list)) {
+                    const int taken = atomicAdd(cursor, 1);
+                    if (taken < in_list) {
+                        chunk = taken * TASK_CURSORS + list;
+                    }
+                }
+            }
+            *(volatile __attribute__((address_space(3))) int *)&lds.next_item = chunk;
+        }
+        group_barrier();
+        const int chunk = __builtin_amdgcn_readfirstlane(*(const volatile __attribute__((address_space(3))) int *)&lds.next_item);
+        if (chunk < 0) {
+            break;
+        }
+        item = chunk * chunk_items;
+        item_end = min(item + chunk_items, items);
     }
     const int task = first_short + item / inner;
     int tile = item % inner;
@@ -560,9 +596,17 @@ TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, c
         }
     }
     group_barrier();   // (the next item reuses the LDS buffers)
+    ++item;
     }
 }
 
+
+// The short groups in a launch of their own (three workgroups of four waves per CU share the items).
+template <int TYPE, bool WIDE>
+__global__ __launch_bounds__(64 * FSS_WAVES, 3) void mmq_forward_scaled_short_kernel(const ForwardArgs a) {
+    __shared__ ShortLds<TYPE> lds;
+    short_group_items<TYPE, WIDE, false>(a, lds, threadIdx.x, 0, gridDim.x);
+}
 
 template <int TYPE, bool WIDE>
 __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(const ForwardArgs a, const int total_slots,
@@ -588,8 +632,8 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
     // the last round of items still occupies the others.
     if (static_cast<int>(blockIdx.x) >= main_blocks) {
         const int group = __builtin_amdgcn_readfirstlane(tid / (64 * FSS_WAVES));
-        short_group_items<TYPE, WIDE>(a, shared.short_groups[group], tid % (64 * FSS_WAVES), group,
-                                      static_cast<int>(gridDim.x) - main_blocks);
+        short_group_items<TYPE, WIDE, true>(a, shared.short_groups[group], tid % (64 * FSS_WAVES), group,
+                                            static_cast<int>(gridDim.x) - main_blocks);
         return;
     }
     L & lds = shared.role_split;
@@ -1212,7 +1256,10 @@ static hipError_t launch_forward_scaled_typed(const ForwardArgs & call, hipStrea
     constexpr int SHORT_GROUPS = FSC_THREADS / (64 * FSS_WAVES);
     const int64_t short_items = args.task_count != nullptr ? static_cast<int64_t>(args.task_slots) * args.n_tiles * args.projections : 0;
     const int64_t short_units = (short_items + SHORT_GROUPS - 1) / SHORT_GROUPS;
-    const int64_t short_blocks = short_units < FSC_GRID ? short_units : FSC_GRID;
+    // (rows of fewer than four super-blocks: the short groups get a launch of their own, see short_group_items)
+    const bool trailing = args.in_features / QK_K >= 4;
+    const int64_t short_blocks = !trailing ? 0 : short_units < FSC_GRID ? short_units : FSC_GRID;
+    const int64_t short_grid = trailing ? 0 : short_items < 3 * FSC_GRID ? short_items : 3 * FSC_GRID;
     if (total <= 0 || total > 0x7fffffffLL || args.swiglu != 0 || args.in_features > (1 << 22)) {
         return hipErrorInvalidValue;
     }
@@ -1238,6 +1285,17 @@ static hipError_t launch_forward_scaled_typed(const ForwardArgs & call, hipStrea
         }
     } else {
         mmq_forward_scaled_kernel<TYPE, false><<<blocks, FSC_THREADS, 0, stream>>>(args, static_cast<int>(total), static_cast<int>(grid));
+    }
+    hipError_t status = hipGetLastError();
+    if (status != hipSuccess || short_grid == 0) {
+        return status;
+    }
+    if (wide) {
+        if constexpr (Format<TYPE>::BLOCK_BYTES % 16 != 0) {
+            mmq_forward_scaled_short_kernel<TYPE, true><<<static_cast<unsigned>(short_grid), 64 * FSS_WAVES, 0, stream>>>(args);
+        }
+    } else {
+        mmq_forward_scaled_short_kernel<TYPE, false><<<static_cast<unsigned>(short_grid), 64 * FSS_WAVES, 0, stream>>>(args);
     }
     return hipGetLastError();
 }

@@ -157,9 +157,12 @@ static inline Q8Workspace q8_workspace_view(void * base, int64_t rows, int64_t i
     return view;
 }
 
-// Tile tasks of the grouped operators: [count][early][expert x max][row_start x max][row_end x max][cursor].
+// Tile tasks of the grouped operators: [count][early][expert x max][row_start x max][row_end x max][cursors].
 // `early` is the number of tasks listed before the short ones (TaskBuild::late_rows); count when nothing is short.
-// `cursor` is zero when the list is built: a kernel whose workgroups take items of the list in turn counts them there.
+// `cursor`: TASK_CURSORS counters, TASK_CURSOR_STRIDE words apart (a cache line each), zero when the list is built: a
+// kernel whose workgroups take items of the list in turn counts them there.
+constexpr int TASK_CURSORS = 8;
+constexpr int TASK_CURSOR_STRIDE = 32;
 struct TaskList {
     int32_t * count;
     int32_t * early;
@@ -176,7 +179,7 @@ static inline int max_tasks_for(int64_t rows, int64_t groups, int row_tile) {
 
 static inline int64_t task_workspace_bytes(int64_t rows, int64_t groups) {
     // sized for the smallest tile any kernel uses so one buffer fits every path
-    return (3 + 3 * static_cast<int64_t>(max_tasks_for(rows, groups, GEMV_ROW_TILE))) *
+    return (2 + 3 * static_cast<int64_t>(max_tasks_for(rows, groups, GEMV_ROW_TILE)) + TASK_CURSOR_STRIDE * (TASK_CURSORS + 1)) *
            static_cast<int64_t>(sizeof(int32_t));
 }
 
@@ -188,7 +191,9 @@ static inline TaskList task_list_view(void * base, int64_t rows, int64_t groups,
     list.expert = list.count + 2;
     list.row_start = list.expert + list.max_tasks;
     list.row_end = list.row_start + list.max_tasks;
-    list.cursor = list.row_end + list.max_tasks;
+    // (the cursors start on a cache line of their own)
+    int32_t * const end = list.row_end + list.max_tasks;
+    list.cursor = end + (TASK_CURSOR_STRIDE - (end - list.count) % TASK_CURSOR_STRIDE) % TASK_CURSOR_STRIDE;
     return list;
 }
 

@@ -1252,7 +1252,7 @@ static hipError_t launch_forward_scaled_typed(const ForwardArgs & call, hipStrea
     const int64_t total = static_cast<int64_t>(args.n_tiles) * args.projections *
                           (args.task_count != nullptr ? xcd_chunk_slots(args.task_slots) : pad_task_slots(args.task_slots, FWD_XCD_RUN));
     // grouped calls: whole groups of at most 32 rows are listed behind the other tasks and go to workgroups of their own,
-    // each of which runs up to three such items at a time (one per CU suffices: they take their items in rounds)
+    // each of which runs up to three such items at a time (one per CU suffices: its groups take items until none is left)
     constexpr int SHORT_GROUPS = FSC_THREADS / (64 * FSS_WAVES);
     const int64_t short_items = args.task_count != nullptr ? static_cast<int64_t>(args.task_slots) * args.n_tiles * args.projections : 0;
     const int64_t short_units = (short_items + SHORT_GROUPS - 1) / SHORT_GROUPS;

@@ -301,3 +301,24 @@ def test_more_tiles_than_one_table_per_cu_holds(ops, grouped):
         a = flat_scaled[begin : begin + step * 16].float()
         b = flat_exact[begin : begin + step * 16].float()
         assert bool(((a - b).abs() <= b.abs() * 2.0**-7 + OPERAND_NOISE["scaled"] * peak).all())
+
+
+@pytest.mark.parametrize("k", (512, 1024))
+@pytest.mark.parametrize("sizes", ([1, 5, 32, 17, 31, 2], [40, 300, 33], [7, 0, 290, 32, 0, 64]))
+def test_only_short_groups_only_long_groups_and_both(ops, oracle, k, sizes):
+    """The scaled kind serves groups of at most 32 rows and the others with different workgroups (of one launch for rows
+    of four super-blocks or more, k = 1024; of two launches below that, k = 512): lists that have only the one kind, only
+    the other, and both with empty groups in between."""
+    tgo, native, synth = ops
+    qtype, n = QTYPES["Q4_K"], 200
+    experts = list(range(len(sizes)))[::-1]
+    offsets = np.cumsum(sizes).tolist()
+    host = synth.random_packed_weight(qtype, (len(sizes), n), k, seed=400 + k)
+    x = random_bf16((offsets[-1], k), seed=401)
+    native.set_forward_operand("scaled")
+    try:
+        actual = tgo.grouped_mmq(x, host.cuda(), *_metadata(experts, offsets), qtype, n)
+    finally:
+        native.set_forward_operand("auto")
+    expected = oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), experts, offsets, n, k, n)
+    assert_matches_f32_reference(actual, expected, OPERAND_NOISE["scaled"])

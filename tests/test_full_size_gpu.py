@@ -53,10 +53,12 @@ def _reverse_within_groups(offsets, rows):
     return torch.from_numpy(index).cuda()
 
 
-def test_pair_forward_and_backward_at_the_benchmark_size(ops, oracle):
-    """256 experts, gate and up Q5_K [512, 2048], 8192 tokens x top-8 with Zipf-skewed routing (65 536 rows)."""
+@pytest.mark.parametrize("qname", ("Q5_K", "IQ2_S"))
+def test_pair_forward_and_backward_at_the_benchmark_size(ops, oracle, qname):
+    """256 experts, gate and up [512, 2048] (Q5_K: the benchmark's format; IQ2_S: the format the reference's model packs
+    them in), 8192 tokens x top-8 with Zipf-skewed routing (65 536 rows)."""
     tgo, synth = ops
-    qtype, n, k, experts = QTYPES["Q5_K"], 512, 2048, 256
+    qtype, n, k, experts = QTYPES[qname], 512, 2048, 256
     token_of_row, indices, offsets, _ = synth.zipf_routing(8192, experts, 8, 2024, device="cuda")
     rows = token_of_row.numel()
     assert rows == 65536

@@ -92,3 +92,38 @@ def test_dense_and_prefill_sized_calls_capture(ops):
             torch.cuda.synchronize()
             for got, expected in zip(captured, eager):
                 assert torch.equal(got, expected)
+
+
+def test_scaled_pair_with_short_groups_replays_bit_identically(ops):
+    """A grouped pair large enough for the scaled operands, with whole groups of at most 32 rows among the others: the
+    launch's trailing workgroups take those from cursors that the quantizer's launch zeroes, so every replay starts
+    from a fresh count."""
+    from torch_ggml_ops import _native
+
+    tgo, synth = ops
+    qtype, n, k, experts = QTYPES["Q5_K"], 512, 1024, 24
+    sizes = [3000, 1, 17, 700, 32, 2500, 9, 260, 31, 1800, 5, 2, 900, 33, 1500]
+    indices = torch.tensor(list(range(len(sizes)))[::-1], device="cuda", dtype=torch.int64)
+    offsets = torch.tensor(sizes, dtype=torch.int64).cumsum(0).to(device="cuda", dtype=torch.int32)
+    rows = int(sum(sizes))
+    assert _native.forward_operand_for(qtype, rows, n, 2) == "scaled"
+    gate = synth.random_packed_weight(qtype, (experts, n), k, 31, device="cuda")
+    up = synth.random_packed_weight(qtype, (experts, n), k, 32, device="cuda")
+    generator = torch.Generator(device="cuda").manual_seed(5)
+    x = torch.randn(rows, k, device="cuda", generator=generator).to(torch.bfloat16)
+
+    def pair():
+        return tgo.grouped_mmq_pair(x, gate, up, indices, offsets, qtype, n)
+
+    eager = [t.clone() for t in pair()]
+    graph, captured = _capture(pair)
+    for replay in range(4):
+        for t in captured:
+            t.zero_()
+        scratch = torch.randn(1 << 16, device="cuda").sum()   # eager work between replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, want in zip(captured, eager):
+            assert torch.equal(got, want), f"replay {replay} differs from the eager result"
+        assert torch.isfinite(scratch)

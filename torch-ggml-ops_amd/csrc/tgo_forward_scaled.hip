@@ -123,20 +123,20 @@ template <int TYPE>
 constexpr int scale_offset() { return TYPE == Q3_K ? 108 : TYPE == Q6_K ? 208 : 0; }
 
 
-// Stores the wave's 32 rows x 128 columns of results, which the matrix instructions left transposed (weights as the
+// Stores the wave's 32 rows x (32 * TILES) columns of results, which the matrix instructions left transposed (weights as the
 // A operand: the lane holds row l32 and, as element v of tile t, column 32 t + 8 (v / 4) + 4 (lane / 32) + v % 4), as
 // bf16.  The two half-waves exchange runs of four columns, after which a lane holds eight neighbouring columns and
 // stores 16 bytes; a row gets 32 contiguous bytes per instruction.  `dst` points at row 0, column 0; rows >=
 // valid_rows and columns >= valid_cols are skipped.  The 16-byte path needs row_stride % 8 == 0 (dst is then 16-byte
 // aligned: the tensor is, and column tiles start at multiples of 128).
-TGO_DEVICE void store_rows_32x128(const v16f (&tiles)[FWD_NT], uint16_t * dst, int64_t row_stride, int valid_rows,
-                                  int valid_cols, int lane) {
+template <int TILES>
+TGO_DEVICE void store_rows_32xn(const v16f * tiles, uint16_t * dst, int64_t row_stride, int valid_rows, int valid_cols, int lane) {
     const int l32 = lane & 31;
     const int half = lane >> 5;
     const bool wide = (row_stride & 7) == 0;
     uint16_t * const row = dst + l32 * row_stride;
 #pragma unroll
-    for (int t = 0; t < FWD_NT; ++t) {
+    for (int t = 0; t < TILES; ++t) {
 #pragma unroll
         for (int m = 0; m < 2; ++m) {
             // runs 2m and 2m + 1 of the tile: the lower half-wave keeps its run 2m and takes the upper one's,
@@ -1221,6 +1221,8 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             asm volatile("" : "+v"(lane_here));
             const int l32_here = lane_here & 31, half_here = lane_here >> 5;
             if (r0 < row_end) {
+                // one column tile at a time, its powers read when they are needed: read for all four tiles ahead of the
+                // stores they no longer fit the registers, and a reload from scratch waits for every store before it
 #pragma unroll
                 for (int nt = 0; nt < FWD_NT; ++nt) {
 #pragma unroll
@@ -1232,9 +1234,10 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
                         acc[nt][4 * j + 2] *= row_power * column_power.z;
                         acc[nt][4 * j + 3] *= row_power * column_power.w;
                     }
+                    store_rows_32xn<1>(&acc[nt], y + static_cast<int64_t>(r0) * a.out_features + n0 + 32 * nt, a.out_features,
+                                       row_end - r0, a.out_features - n0 - 32 * nt, lane_here);
+                    __builtin_amdgcn_sched_barrier(0);
                 }
-                store_rows_32x128(acc, y + static_cast<int64_t>(r0) * a.out_features + n0, a.out_features, row_end - r0,
-                                  a.out_features - n0, lane_here);
             }
 #pragma unroll
             for (int nt = 0; nt < FWD_NT; ++nt) acc[nt] = zero;

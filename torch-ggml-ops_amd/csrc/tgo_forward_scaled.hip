@@ -690,24 +690,31 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             *(SharedCounter)counter = value;
         }
     };
+    // (counts only grow: what a poll has seen serves every later wait that it already satisfies, without touching LDS,
+    // whose queue a poll has to drain first)
+    int seen_produced = 0, seen_consumed = 0;
     auto wait_produced = [&](int need) __attribute__((always_inline)) {
-        for (int polls = 0; polls < FSC_SPIN_LIMIT; ++polls) {
-            const i32x4_t v = *(SharedCounters)&lds.produced[0];
-            if (__builtin_amdgcn_readfirstlane(min(min(v.x, v.y), min(v.z, v.w))) >= need) {
-                break;
+        if (seen_produced < need) {
+            for (int polls = 0; polls < FSC_SPIN_LIMIT; ++polls) {
+                const i32x4_t v = *(SharedCounters)&lds.produced[0];
+                seen_produced = __builtin_amdgcn_readfirstlane(min(min(v.x, v.y), min(v.z, v.w)));
+                if (seen_produced >= need) {
+                    break;
+                }
+                __builtin_amdgcn_s_sleep(1);
             }
-            __builtin_amdgcn_s_sleep(1);
         }
         asm volatile("" ::: "memory");   // (the data accesses stay after the count)
     };
     auto wait_consumed = [&](int need) __attribute__((always_inline)) {
         static_assert(FSC_MULTIPLIERS == 8, "two 16-byte reads cover the multipliers' counters");
-        if (need > 0) {
+        if (seen_consumed < need) {
             for (int polls = 0; polls < FSC_SPIN_LIMIT; ++polls) {
                 const i32x4_t v = *(SharedCounters)&lds.consumed[0];
                 const i32x4_t u = *(SharedCounters)&lds.consumed[4];
                 const int least = min(min(min(v.x, v.y), min(v.z, v.w)), min(min(u.x, u.y), min(u.z, u.w)));
-                if (__builtin_amdgcn_readfirstlane(least) >= need) {
+                seen_consumed = __builtin_amdgcn_readfirstlane(least);
+                if (seen_consumed >= need) {
                     break;
                 }
                 __builtin_amdgcn_s_sleep(1);

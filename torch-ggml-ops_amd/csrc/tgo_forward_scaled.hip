@@ -371,6 +371,9 @@ TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, c
     const uint8_t * const sums_base = reinterpret_cast<const uint8_t *>(a.block_sums) + static_cast<int64_t>(first_tile) * super_blocks * 512;
     int lane_row = row_start + l32;
     lane_row = lane_row < a.rows_padded ? lane_row : a.rows_padded - 1;
+    // 2^E of the lane's row, for the epilogue (requested here: asked for there, the whole item would wait for it, and
+    // for every load still in flight in front of it)
+    const float row_power = a.row_power[lane_row];
     const uint32_t x_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * blocks_per_row * 2048u +
                             static_cast<uint32_t>(((lane_row & 31) + 32 * half) * 16);
     const uint32_t sums_lane = static_cast<uint32_t>((lane_row >> 5) - first_tile) * super_blocks * 512u +
@@ -561,39 +564,16 @@ TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, c
 
     // ---- epilogue: scale by 2^(E[r] + S[n]) and store 32 rows x 32 columns
     {
-        const float row_power = a.row_power[lane_row];
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             acc[v] = total[v] * row_power;
         }
         uint16_t * const y = (second ? a.y_second : a.y) + static_cast<int64_t>(row_start) * a.out_features + n0;
-        const bool wide_rows = (a.out_features & 7) == 0;
-        uint16_t * const row = y + l32 * static_cast<int64_t>(a.out_features);
-        const int valid_rows = row_end - row_start;
-        const int valid_cols = a.out_features - n0;
-#pragma unroll
-        for (int m = 0; m < 2; ++m) {
-            const uint32_t p0 = pack_bf16x2(acc[8 * m + 0], acc[8 * m + 1]);
-            const uint32_t p1 = pack_bf16x2(acc[8 * m + 2], acc[8 * m + 3]);
-            const uint32_t q0 = pack_bf16x2(acc[8 * m + 4], acc[8 * m + 5]);
-            const uint32_t q1 = pack_bf16x2(acc[8 * m + 6], acc[8 * m + 7]);
-            const auto s0 = __builtin_amdgcn_permlane32_swap(p0, q0, false, false);
-            const auto s1 = __builtin_amdgcn_permlane32_swap(p1, q1, false, false);
-            const uint32_t words[4] = {s0[0], s1[0], s0[1], s1[1]};
-            const int c = 16 * m + 8 * half;
-            if (l32 < valid_rows && c < valid_cols) {
-                if (wide_rows && c + 8 <= valid_cols) {
-                    *reinterpret_cast<uint4 *>(row + c) = make_uint4(words[0], words[1], words[2], words[3]);
-                } else {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) {
-                        if (c + e < valid_cols) {
-                            row[c + e] = static_cast<uint16_t>(words[e >> 1] >> (16 * (e & 1)));
-                        }
-                    }
-                }
-            }
-        }
+        // (recomputing the lane's share here is cheaper than keeping it alive through the loop: kept, it is spilled, and
+        // its reload waits for every load in flight)
+        int lane_here = lane;
+        asm volatile("" : "+v"(lane_here));
+        store_rows_32xn<1>(&acc, y, a.out_features, row_end - row_start, a.out_features - n0, lane_here);
     }
     group_barrier();   // (the next item reuses the LDS buffers)
     ++item;

@@ -129,6 +129,14 @@ constexpr int scale_offset() { return TYPE == Q3_K ? 108 : TYPE == Q6_K ? 208 : 
 // stores 16 bytes; a row gets 32 contiguous bytes per instruction.  `dst` points at row 0, column 0; rows >=
 // valid_rows and columns >= valid_cols are skipped.  The 16-byte path needs row_stride % 8 == 0 (dst is then 16-byte
 // aligned: the tensor is, and column tiles start at multiples of 128).
+// The lane's number computed from nothing, and opaque: what is derived from it is derived where it is used instead of
+// being kept in a register through a loop (where such a register is spilled, its reload waits for every load in flight).
+TGO_DEVICE int lane_afresh() {
+    int lane = static_cast<int>(__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)));
+    asm volatile("" : "+v"(lane));
+    return lane;
+}
+
 template <int TILES>
 TGO_DEVICE void store_rows_32xn(const v16f * tiles, uint16_t * dst, int64_t row_stride, int valid_rows, int valid_cols, int lane) {
     const int l32 = lane & 31;
@@ -571,8 +579,7 @@ TGO_DEVICE void short_group_items(const ForwardArgs & a, ShortLds<TYPE> & lds, c
         uint16_t * const y = (second ? a.y_second : a.y) + static_cast<int64_t>(row_start) * a.out_features + n0;
         // (recomputing the lane's share here is cheaper than keeping it alive through the loop: kept, it is spilled, and
         // its reload waits for every load in flight)
-        int lane_here = lane;
-        asm volatile("" : "+v"(lane_here));
+        const int lane_here = lane_afresh();
         store_rows_32xn<1>(&acc, y, a.out_features, row_end - row_start, a.out_features - n0, lane_here);
     }
     group_barrier();   // (the next item reuses the LDS buffers)
@@ -1204,8 +1211,7 @@ __global__ __launch_bounds__(FSC_THREADS, 3) void mmq_forward_scaled_kernel(cons
             uint16_t * const y = second ? a.y_second : a.y;
             const int r0 = row_start + wave * 32;
             // recomputing the lane's share here is cheaper than keeping it alive through the loop
-            int lane_here = lane;
-            asm volatile("" : "+v"(lane_here));
+            const int lane_here = lane_afresh();
             const int l32_here = lane_here & 31, half_here = lane_here >> 5;
             if (r0 < row_end) {
                 // one column tile at a time, its powers read when they are needed: read for all four tiles ahead of the

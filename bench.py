@@ -209,6 +209,7 @@ def measure_decode(args, device) -> dict:
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - start
         kernel_ms, launches = _native.profile_read("forward_gemv")
+        quantize_ms, _ = _native.profile_read("quantize")   # (zero where the GEMV kernels quantize their own rows)
         _native.lib.tgo_profile_enable(0)
         if launches == 0:
             continue  # too many rows per expert for the GEMV family: that shape belongs to the MFMA benchmark
@@ -239,6 +240,8 @@ def measure_decode(args, device) -> dict:
             "us_per_layer_call_graph_replay": graph_elapsed / args.steps * 1e6,
             "GBps_end_to_end": weight_bytes / (elapsed / args.steps) / 1e9,
             "gemv_kernel_us_per_step": kernel_ms / args.steps * 1e3,
+            "quantize_kernel_us_per_step": quantize_ms / args.steps * 1e3,
+            "launches_per_layer_call": launches / args.steps + (2 if quantize_ms > 0 else 0),
             "GBps_gemv_kernels": weight_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
         }
     x = torch.randn(1, 2048, device=device, generator=generator).to(torch.bfloat16)

@@ -146,3 +146,72 @@ def test_skewed_small_batch_listed_with_every_expert(ops, oracle, qname):
     compact = tgo.grouped_mmq(x, host.cuda(), torch.tensor(listed, dtype=torch.int64, device="cuda"),
                               torch.tensor(np.cumsum([sizes[e] for e in listed]).tolist(), dtype=torch.int32, device="cuda"), qtype, n)
     assert_matches_f32_reference(compact, expected)
+
+
+@pytest.mark.parametrize("qname", ("IQ2_S", "Q6_K", "Q3_K"))
+def test_grouped_decode_finds_tasks_among_many_groups(ops, oracle, qname):
+    """Small grouped calls of these formats are one launch whose workgroups look their task up in the group list
+    themselves, 256 groups per round: 700 listed groups (nearly all empty, some with more than one task, some naming an
+    expert that does not exist) make the lookup run three rounds, with tasks on both sides of every round's boundary."""
+    tgo, native, synth = ops
+    qtype, n, k, experts = QTYPES[qname], 40, 512, 700
+    rng = np.random.default_rng(77 + qtype)
+    sizes = np.zeros(experts, dtype=np.int64)
+    for group, size in ((0, 9), (100, 1), (254, 2), (255, 3), (256, 1), (257, 8), (300, 4), (511, 2), (512, 10),
+                        (513, 1), (600, 5), (699, 3)):
+        sizes[group] = size
+    chosen = rng.permutation(experts)
+    unknown = [100, 255, 300, 513]
+    chosen[unknown] = [experts, experts + 7, -1, 10**9]
+    offsets = np.cumsum(sizes).tolist()
+    rows = offsets[-1]
+    assert rows <= 64 and native.lib.tgo_forward_kernel_family(rows, experts) == b"gemv"
+    host = synth.random_packed_weight(qtype, (experts, n), k, seed=55 + qtype)
+    x = random_bf16((rows, k), seed=19)
+    actual = tgo.grouped_mmq(x, host.cuda(), torch.tensor(chosen, dtype=torch.int64, device="cuda"),
+                             torch.tensor(offsets, dtype=torch.int32, device="cuda"), qtype, n)
+    exact = oracle.grouped(oracle.mmq_forward, qtype, bits(x), host.numpy(), chosen.tolist(), offsets, n, k, n)
+    covered = ~np.isnan(exact[:, 0])
+    assert covered.sum() == rows - sum(int(sizes[g]) for g in unknown)
+    assert_matches_f32_reference(actual[torch.from_numpy(covered).cuda()], exact[covered])
+
+
+@pytest.mark.parametrize("qname", ("IQ2_S", "Q6_K", "Q3_K"))
+@pytest.mark.parametrize("rows", (15, 64, 72))
+def test_one_launch_and_two_launch_decode_agree(ops, qname, rows):
+    """Calls of at most 8 (dense) or 64 (grouped) rows quantize inside the decode kernels, larger ones in a launch of
+    their own; the arithmetic is the same, so a call split into small ones gives the same bits."""
+    tgo, _, synth = ops
+    qtype, n, k, experts = QTYPES[qname], 48, 2304, 24
+    weight = synth.random_packed_weight(qtype, (experts, n), k, seed=61 + qtype).cuda()
+    x = random_bf16((rows, k), seed=rows)
+    sizes = np.full(experts, rows // experts)
+    sizes[: rows % experts] += 1
+    indices = torch.arange(experts, dtype=torch.int64, device="cuda")
+    whole = tgo.grouped_mmq(x, weight, indices, torch.tensor(np.cumsum(sizes), dtype=torch.int32, device="cuda"), qtype, n)
+    begin = 0
+    for expert, size in enumerate(sizes.tolist()):
+        if size == 0:   # (an empty group is legal, a dense call without rows is not)
+            continue
+        part = tgo.mmq(x[begin:begin + size].clone(), weight[expert].clone(), qtype, n)
+        torch.testing.assert_close(whole[begin:begin + size], part, rtol=0, atol=0)
+        begin += size
+
+
+@pytest.mark.parametrize("qname", ("IQ2_S", "Q6_K"))
+def test_gathered_decode_reads_absent_rows_as_zeros(ops, qname):
+    """The decode kernels that quantize their own activations gather them too: an index outside the token range is a
+    row of zeros, and every other row equals the plain call on the gathered rows bit for bit."""
+    tgo, _, synth = ops
+    qtype, n, k = QTYPES[qname], 48, 2304
+    weight = synth.random_packed_weight(qtype, (3, n), k, seed=41).cuda()
+    hidden = random_bf16((4, k), seed=42)
+    row_index = torch.tensor([2, -1, 0, 9, 3, 1], device="cuda", dtype=torch.int64)
+    indices = torch.tensor([0, 2], device="cuda", dtype=torch.int64)
+    offsets = torch.tensor([2, 6], device="cuda", dtype=torch.int32)
+    out = tgo.grouped_mmq_gathered(hidden, row_index, weight, indices, offsets, qtype, n)
+    padded = torch.cat([hidden, torch.zeros_like(hidden[:1])])
+    safe = torch.tensor([2, 4, 0, 4, 3, 1], device="cuda")
+    expected = tgo.grouped_mmq(padded.index_select(0, safe), weight, indices, offsets, qtype, n)
+    torch.testing.assert_close(out, expected, rtol=0, atol=0)
+    assert torch.count_nonzero(out[1]) == 0 and torch.count_nonzero(out[3]) == 0

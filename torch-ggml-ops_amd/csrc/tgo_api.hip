@@ -330,6 +330,15 @@ int tgo_mmq_forward(const void * input_bf16, const void * packed, void * output_
     TGO_TRY(check_pointer(output_bf16, "output"));
     TGO_TRY(check_pointer(workspace, "workspace"));
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
+    if (tgo::gemv_fuses(quant_type, rows, 0)) {
+        // one launch: the decode-regime kernels of these formats quantize their activations themselves
+        return check_hip(tgo::launch_mmq_gemv_fused(static_cast<const uint8_t *>(packed), nullptr, 0,
+                                                    static_cast<const uint16_t *>(input_bf16), nullptr, rows, nullptr,
+                                                    nullptr, 0, 0, static_cast<uint16_t *>(output_bf16), nullptr,
+                                                    static_cast<int>(rows), static_cast<int>(in_features),
+                                                    static_cast<int>(out_features), quant_type, hip_stream),
+                         "mmq_forward launch");
+    }
     const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, tgo::use_gemv(rows, 0),
                                                          tgo::forward_operand_kind(quant_type, rows, out_features, 1));
     TGO_TRY(check_hip(tgo::launch_quantize_q8_1(static_cast<const uint16_t *>(input_bf16), view, rows, in_features,
@@ -439,6 +448,19 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
     const int64_t bytes_per_expert = out_features * (in_features / tgo::QK_K) * tgo::block_bytes(quant_type);
     // (the fused SwiGLU epilogue exists in the MFMA kernel only)
     const bool gemv = !swiglu && tgo::use_gemv(rows, num_groups);
+    if (gemv && tgo::gemv_fuses(quant_type, rows, num_groups)) {
+        // one launch: the decode-regime kernels of these formats quantize their activations and find their tasks
+        // themselves
+        return check_hip(tgo::launch_mmq_gemv_fused(
+                             static_cast<const uint8_t *>(packed_first), static_cast<const uint8_t *>(packed_second),
+                             bytes_per_expert, static_cast<const uint16_t *>(input_bf16), row_index,
+                             row_index != nullptr ? input_rows : rows, expert_indices, expert_offsets,
+                             static_cast<int>(num_experts), static_cast<int>(num_groups),
+                             static_cast<uint16_t *>(output_first), static_cast<uint16_t *>(output_second),
+                             static_cast<int>(rows), static_cast<int>(in_features), static_cast<int>(out_features),
+                             quant_type, hip_stream),
+                         "grouped mmq_forward launch");
+    }
     const int operand_kind = tgo::forward_operand_kind(quant_type, rows, out_features, packed_second != nullptr ? 2 : 1);
     // the scaled-operand kernel has no SwiGLU epilogue: it stores both projections (the up projection where the
     // result goes) and an elementwise pass finishes, which costs less than the other kinds' kernels lose to it

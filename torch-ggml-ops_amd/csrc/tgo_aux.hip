@@ -68,72 +68,8 @@ int forward_operand_setting() { return g_forward_operand.load(std::memory_order_
 void set_forward_operand_setting(int operand) { g_forward_operand.store(operand, std::memory_order_relaxed); }
 
 // ---- bf16 activations -> q8_1 -------------------------------------------------------------------
-// Arithmetic of the reference quantizer (csrc/mmq_core.cuh:151-209): per 32 values amax, d = amax/127,
-// q = roundf(x * (127/amax)), and the fp32 sum of the values added in the reference's order (four per
-// lane left to right, then a butterfly over eight lanes with offsets 4, 2, 1).  Here a lane holds eight
-// values, i.e. two of the reference's lanes, so the butterfly runs over four lanes on two partial sums.
-// One workgroup handles 32 rows x 256 values and writes one contiguous 8 KiB run of fragment-ordered int8.
-// Eight consecutive values of a 32-value block per lane (four neighbouring lanes hold the block): the block's
-// scale, the lane's eight int8 values and the block's sum, the same on all four lanes.
-// round(v) to the nearest integer, halves away from zero (roundf), of a magnitude: the hardware's
-// round-to-nearest-with-ties-up conversion of |v| is exactly that for non-negative inputs.
-TGO_DEVICE int round_magnitude(float v) {
-    int magnitude;
-    asm("v_cvt_rpi_i32_f32 %0, |%1|" : "=v"(magnitude) : "v"(v));
-    return magnitude;
-}
-
-// `bits` are the lane's eight bf16 values as loaded (two per word), `x` the same as floats.  The quants are
-// formed as magnitudes, two per register as 16-bit integers, and get their signs from the bf16 words themselves
-// (an arithmetic shift of each half by 15 is the sign mask of the value it holds): (m ^ s) - s with packed 16-bit
-// operations, then one byte permute per four values.
-typedef short short2_t __attribute__((ext_vector_type(2)));
-// `halves`: the same quants as fp16 numbers, two per register (1024 + magnitude is the magnitude placed under the
-// bits of 1024.0; the sign bit is the one of the bf16 value, which sits at the same place of its half-word).
-// `magnitude`: |q| of the eight values (for the scaled layout, which stores d * q instead of q).
-TGO_DEVICE void quantize_eight(const uint4 bits, const float (&x)[8], uint32_t (&packed)[2], float & d, float & total,
-                               uint32_t (&halves)[4], int (&magnitude)[8]) {
-    float amax = fmaxf(fmaxf(fabsf(x[0]), fabsf(x[1])), fabsf(x[2]));
-    amax = fmaxf(fmaxf(amax, fabsf(x[3])), fabsf(x[4]));
-    amax = fmaxf(fmaxf(amax, fabsf(x[5])), fabsf(x[6]));
-    amax = fmaxf(amax, fabsf(x[7]));
-    amax = fmaxf(amax, __shfl_xor(amax, 1));
-    amax = fmaxf(amax, __shfl_xor(amax, 2));
-
-    float even = ((x[0] + x[1]) + x[2]) + x[3];
-    float odd = ((x[4] + x[5]) + x[6]) + x[7];
-    even = even + __shfl_xor(even, 2);
-    odd = odd + __shfl_xor(odd, 2);
-    even = even + __shfl_xor(even, 1);
-    odd = odd + __shfl_xor(odd, 1);
-    total = even + odd;
-
-    d = amax == 0.0f ? 0.0f : amax / 127.0f;
-    const float d_inv = amax == 0.0f ? 0.0f : 127.0f / amax;
-    const uint32_t words[4] = {bits.x, bits.y, bits.z, bits.w};
-    uint32_t signed_pairs[4];
-#pragma unroll
-    for (int pair = 0; pair < 4; ++pair) {
-        magnitude[2 * pair] = round_magnitude(x[2 * pair] * d_inv);
-        magnitude[2 * pair + 1] = round_magnitude(x[2 * pair + 1] * d_inv);
-        const short2_t magnitudes = __builtin_amdgcn_cvt_pk_i16(magnitude[2 * pair], magnitude[2 * pair + 1]);
-        const short2_t sign = __builtin_bit_cast(short2_t, words[pair]) >> 15;
-        signed_pairs[pair] = __builtin_bit_cast(uint32_t, static_cast<short2_t>((magnitudes ^ sign) - sign));
-        halves[pair] = half2_add(__builtin_bit_cast(uint32_t, magnitudes) | 0x64006400u, half2_of(-1024)) |
-                       (words[pair] & 0x80008000u);
-    }
-    // low byte of each 16-bit half: bytes 0 and 2 of the first word, then of the second
-    packed[0] = __builtin_amdgcn_perm(signed_pairs[1], signed_pairs[0], 0x06040200u);
-    packed[1] = __builtin_amdgcn_perm(signed_pairs[3], signed_pairs[2], 0x06040200u);
-}
-
-TGO_DEVICE void unpack_bf16x8(const uint4 bits, float (&x)[8]) {
-    x[0] = bf16_bits_to_float(bits.x & 0xffffu); x[1] = bf16_bits_to_float(bits.x >> 16);
-    x[2] = bf16_bits_to_float(bits.y & 0xffffu); x[3] = bf16_bits_to_float(bits.y >> 16);
-    x[4] = bf16_bits_to_float(bits.z & 0xffffu); x[5] = bf16_bits_to_float(bits.z >> 16);
-    x[6] = bf16_bits_to_float(bits.w & 0xffffu); x[7] = bf16_bits_to_float(bits.w >> 16);
-}
-
+// The arithmetic is quantize_eight's (tgo_device.h).  The tile layouts: one workgroup handles 32 rows x 256 values and
+// writes one contiguous 8 KiB run of fragment-ordered int8.
 // Row-major variant for calls that take the GEMV kernels (a handful of rows): workgroup = one row x 2048 values.
 __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t * __restrict__ input,
                                                                 int8_t * __restrict__ q_out,

@@ -50,7 +50,22 @@ struct GemvArgs {
     int n_groups;   // workgroups per task and projection: groups of GEMV_GN (long) weight rows
     int projections;   // 1, or 2 for a pair
     int unit_staging;  // 2-byte aligned formats: the tensors may be read in whole aligned 16-byte units (wide_stage_ok)
+    // Fused calls (kernel instances with FUSED set): the activations arrive as bf16 and every workgroup quantizes the
+    // rows of its task itself, so that a call is one launch; qx, dx, sx and the task arrays are not used.
+    const uint16_t * x;              // [input_rows or rows, in_features] bf16
+    const int64_t * gather;          // row r of the call is row gather[r] of x (absent when outside [0, input_rows)), or nullptr
+    int64_t input_rows;
+    const int64_t * expert_indices;  // grouped fused calls: the groups themselves (a workgroup finds its task in them)
+    const int32_t * expert_offsets;
+    int num_experts;
+    int num_groups;
 };
+
+// LDS of a fused workgroup's activations: ROWS rows of a pass's int8 values, then ROWS x 64 block scales.
+template <int ROWS>
+constexpr int gemv_fused_x_bytes() {
+    return ROWS * GEMV_CHUNK * QK_K + ROWS * GEMV_CHUNK * 8 * 4;
+}
 
 // LDS slot of super-block `kb` of a pass for weight row `row`.  Row-major, so that the lanes of a wave, which
 // differ in kb, hit slots one RAW_PITCH (an odd number of words) apart and spread over the banks; with the
@@ -398,8 +413,12 @@ TGO_DEVICE void gemv_unit(const uint8_t * blk, int u, const uint2 * grid, uint32
 // differs: its unit belongs to weight row `sub` of the long row (FOLD 2: the slot; FOLD 4: slot and half of the
 // wave), the activations repeat with the real K, and the partial sums are kept per slot and reduced over the lanes
 // that share a weight row.  n0 counts long rows; out_features must be a multiple of FOLD.
-template <int TYPE, int ROWS, int FOLD>
-TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid, const uint8_t * weights,
+//
+// FUSED: the activations are bf16 in memory; before a pass's weights are staged every thread requests eight values of
+// each of the task's rows, and while the weights travel it quantizes them (quantize_eight, the quantizer kernels'
+// arithmetic, so the results are the same bit for bit) into x_lds, where the pass reads them after its barrier.
+template <int TYPE, int ROWS, int FOLD, bool FUSED>
+TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, uint8_t * x_lds, const uint2 * grid, const uint8_t * weights,
                           uint16_t * y, int n0, int row_start, int nrows, int tid) {
     using F = Format<TYPE>;
     static_assert(FOLD == 1 || FOLD == 2 || FOLD == 4, "long rows of one, two or four weight rows");
@@ -429,11 +448,13 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
     // of one or two rows request both units before the pass's weights are staged, so that everything travels
     // together; with more rows the registers are needed elsewhere and a unit's activations are fetched when its
     // turn comes.
-    constexpr bool EARLY = ROWS <= 2;
+    constexpr bool EARLY = ROWS <= 2 && !FUSED;
     struct Activations {
         uint4 q[ROWS];
         float d[ROWS];
     };
+    int8_t * const xq_lds = reinterpret_cast<int8_t *>(x_lds);
+    float * const xd_lds = reinterpret_cast<float *>(x_lds + ROWS * GEMV_CHUNK * QK_K);
     auto load_activations = [&](int kb0, int slot, Activations & x) {
         const int unit_in_chunk = lane + 64 * slot;
         // lanes past the end repeat the last block
@@ -443,12 +464,34 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
         const int half = unit & 1;
 #pragma unroll
         for (int r = 0; r < ROWS; ++r) {
-            const int row = row_start + (r < nrows ? r : nrows - 1);
-            x.q[r] = *reinterpret_cast<const uint4 *>(
-                a.qx + static_cast<int64_t>(row) * a.in_features + block * 32 + half * 16);
-            x.d[r] = a.dx[static_cast<int64_t>(row) * blocks_per_row + block];
+            if constexpr (FUSED) {
+                // (the pass's copy in LDS starts at super-block kb0; rows the task does not have were written as zeros)
+                const int local = block - kb0 * 8;
+                x.q[r] = *reinterpret_cast<const uint4 *>(xq_lds + r * GEMV_CHUNK * QK_K + local * 32 + half * 16);
+                x.d[r] = xd_lds[r * GEMV_CHUNK * 8 + local];
+            } else {
+                const int row = row_start + (r < nrows ? r : nrows - 1);
+                x.q[r] = *reinterpret_cast<const uint4 *>(
+                    a.qx + static_cast<int64_t>(row) * a.in_features + block * 32 + half * 16);
+                x.d[r] = a.dx[static_cast<int64_t>(row) * blocks_per_row + block];
+            }
         }
     };
+    // FUSED: where the task's rows are in x (nullptr: a gathered row that does not exist, quantized as zeros)
+    const uint16_t * x_row[FUSED ? ROWS : 1];
+    if constexpr (FUSED) {
+#pragma unroll
+        for (int r = 0; r < ROWS; ++r) {
+            const int row = row_start + (r < nrows ? r : nrows - 1);
+            int64_t source = row;
+            bool present = true;
+            if (a.gather != nullptr) {
+                source = a.gather[row];
+                present = source >= 0 && source < a.input_rows;
+            }
+            x_row[r] = present ? a.x + source * a.in_features : nullptr;
+        }
+    }
 
     for (int kb0 = 0; kb0 < long_blocks; kb0 += GEMV_CHUNK) {
         const int chunk_blocks = min(GEMV_CHUNK, long_blocks - kb0);
@@ -457,7 +500,21 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
             load_activations(kb0, 0, early[0]);
             load_activations(kb0, 1, early[1]);
         }
-        __syncthreads();   // the previous pass is done with `raw`
+        // FUSED: this thread's eight values of the pass for every row (a pass covers the real K once, also for long
+        // rows), requested ahead of the weights
+        const int x_k = (FOLD == 1 ? kb0 * QK_K : 0) + tid * 8;
+        const bool x_mine = tid * 8 < (FOLD == 1 ? chunk_blocks : super_blocks) * QK_K;   // (whole blocks of four lanes)
+        uint4 x_bits[FUSED ? ROWS : 1];
+        if constexpr (FUSED) {
+#pragma unroll
+            for (int r = 0; r < ROWS; ++r) {
+                x_bits[r] = make_uint4(0, 0, 0, 0);
+                if (r < nrows && x_mine && x_row[r] != nullptr) {
+                    x_bits[r] = *reinterpret_cast<const uint4 *>(x_row[r] + x_k);
+                }
+            }
+        }
+        __syncthreads();   // the previous pass is done with `raw` (and with the activations in LDS)
         if (unit_staging) {
             gemv_stage_units<TYPE>(raw, weights + static_cast<int64_t>(n0) * long_row_bytes, long_row_bytes,
                                    min(GEMV_GN, long_rows - n0), kb0, chunk_blocks, tid);
@@ -467,6 +524,27 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, const uint2 * grid,
             gemv_stage_pieces<TYPE, 4>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
         } else {
             gemv_stage<TYPE>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
+        }
+        if constexpr (FUSED) {
+            if (x_mine) {
+#pragma unroll
+                for (int r = 0; r < ROWS; ++r) {
+                    // (rows past the task's last are all zeros: d = 0 and q = 0, no arithmetic needed)
+                    uint32_t packed[2] = {0u, 0u};
+                    float d = 0.0f;
+                    if (r < nrows) {   // uniform
+                        float x[8], total;
+                        uint32_t halves[4];
+                        int magnitude[8];
+                        unpack_bf16x8(x_bits[r], x);
+                        quantize_eight(x_bits[r], x, packed, d, total, halves, magnitude);
+                    }
+                    *reinterpret_cast<uint2 *>(xq_lds + r * GEMV_CHUNK * QK_K + tid * 8) = make_uint2(packed[0], packed[1]);
+                    if ((tid & 3) == 0) {
+                        xd_lds[r * GEMV_CHUNK * 8 + (tid >> 2)] = d;
+                    }
+                }
+            }
         }
         __syncthreads();
 
@@ -1178,9 +1256,10 @@ TGO_DEVICE void gemv_task_k45_mfma(const GemvArgs & a, uint8_t * raw, float * sc
     }
 }
 
-template <int TYPE, int ROWS, int FOLD>
+template <int TYPE, int ROWS, int FOLD, bool FUSED>
 TGO_DEVICE void gemv_rows(const GemvArgs & a, uint8_t * raw, float * scale_lds, uint8_t * x_lds, const uint2 * grid,
                           const uint8_t * weights, uint16_t * y, int n0, int row_start, int nrows, int tid) {
+    static_assert(!FUSED || (TYPE != Q4_K && TYPE != Q5_K), "the Q4_K / Q5_K routines read quantized activations");
     if constexpr ((TYPE == Q4_K || TYPE == Q5_K) && ROWS > 2) {
         // (no long rows in the matrix-core routine: it takes the 16 * FOLD weight rows 16 at a time)
         if constexpr (FOLD == 1) {
@@ -1205,8 +1284,68 @@ TGO_DEVICE void gemv_rows(const GemvArgs & a, uint8_t * raw, float * scale_lds, 
     if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
         gemv_task_k45<TYPE, ROWS <= 2 ? ROWS : 1, FOLD>(a, raw, weights, y, n0, row_start, nrows, tid);
     } else {
-        gemv_task<TYPE, ROWS, FOLD>(a, raw, grid, weights, y, n0, row_start, nrows, tid);
+        gemv_task<TYPE, ROWS, FOLD, FUSED>(a, raw, x_lds, grid, weights, y, n0, row_start, nrows, tid);
     }
+}
+
+// Fused grouped calls: task `task` of the list that build_tasks would write for row tiles of GEMV_ROWS (group g covers
+// rows [offsets[g - 1], offsets[g]) of expert indices[g]; groups with an expert out of range, no rows or rows outside
+// the input are dropped; every other group is cut into tasks of at most GEMV_ROWS rows, in group order), found by the
+// workgroup itself: 256 groups per round, a prefix sum of their task counts, and the thread whose group holds the
+// task publishes it.  All threads of the workgroup call this; false when the list has no such task.
+TGO_DEVICE bool gemv_find_task(const GemvArgs & a, int task, int tid, int * shared, int & expert, int & row_start,
+                               int & row_end) {
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    if (tid == 0) {
+        shared[4] = -1;
+    }
+    int running = 0;   // tasks of the groups of earlier rounds (the same on every thread)
+    for (int base = 0; base < a.num_groups; base += GEMV_THREADS) {
+        const int group = base + tid;
+        int begin = 0, end = 0, group_expert = -1, count = 0;
+        if (group < a.num_groups) {
+            begin = group == 0 ? 0 : a.expert_offsets[group - 1];
+            end = a.expert_offsets[group];
+            const int64_t expert64 = a.expert_indices[group];
+            if (expert64 >= 0 && expert64 < a.num_experts && begin >= 0 && end > begin && end <= a.rows) {
+                group_expert = static_cast<int>(expert64);
+                count = (end - begin + GEMV_ROWS - 1) / GEMV_ROWS;
+            }
+        }
+        int inclusive = count;
+#pragma unroll
+        for (int offset = 1; offset < 64; offset <<= 1) {
+            const int below = __shfl_up(inclusive, offset);
+            inclusive += lane >= offset ? below : 0;
+        }
+        __syncthreads();   // (the previous round's wave totals have been read)
+        if (lane == 63) {
+            shared[wave] = inclusive;
+        }
+        __syncthreads();
+        int before = running;
+#pragma unroll
+        for (int w = 0; w < GEMV_THREADS / 64; ++w) {
+            const int total = shared[w];
+            before += w < wave ? total : 0;
+            running += total;
+        }
+        const int first = before + inclusive - count;
+        if (task >= first && task < first + count) {
+            shared[4] = group_expert;
+            shared[5] = begin + (task - first) * GEMV_ROWS;
+            shared[6] = end;
+        }
+        if (running > task) {   // uniform
+            break;
+        }
+    }
+    __syncthreads();
+    expert = shared[4];
+    row_start = shared[5];
+    row_end = min(row_start + GEMV_ROWS, shared[6]);
+    return expert >= 0;
 }
 
 // MAX_ROWS (1, 2, 4 or 8) bounds the rows of any task of the launch: the register budget, and with it how
@@ -1215,7 +1354,9 @@ TGO_DEVICE void gemv_rows(const GemvArgs & a, uint8_t * raw, float * scale_lds, 
 // WALK: a dense call of more than GEMV_ROWS rows, taken GEMV_ROWS at a time.  Its own instantiation: around that
 // loop the compiler keeps the routines' per-thread constants in registers, which costs the single-pass kernels
 // (every grouped call, every dense call of up to GEMV_ROWS rows) a wave per SIMD if they share the code.
-template <int TYPE, int MAX_ROWS, int FOLD, bool WALK = false>
+// FUSED: bf16 activations, quantized by the workgroups themselves (gemv_task), and, for grouped calls, the task looked
+// up in the group list instead of a task list (gemv_find_task): the whole call is this one launch.
+template <int TYPE, int MAX_ROWS, int FOLD, bool WALK = false, bool FUSED = false>
 __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a) {
     static_assert(!WALK || MAX_ROWS == GEMV_ROWS, "a walked call has full chunks");
     using F = Format<TYPE>;
@@ -1225,7 +1366,10 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a
     constexpr bool TABLES = (TYPE == Q4_K || TYPE == Q5_K) && MAX_ROWS > 2;
     __shared__ __attribute__((aligned(16))) float scale_lds[TABLES ? 2 * (GEMV_THREADS / 64) * GEMV_CHUNK * GEMV_K45_KB_SCALES : 4];
     // its copy of a pass's activations: q8_1 values, block scales, block sums
-    __shared__ __attribute__((aligned(16))) uint8_t x_lds[TABLES ? GEMV_ROWS * GEMV_X_PITCH + 2 * GEMV_ROWS * GEMV_XD_PITCH * 4 : 16];
+    __shared__ __attribute__((aligned(16))) uint8_t x_lds[TABLES  ? GEMV_ROWS * GEMV_X_PITCH + 2 * GEMV_ROWS * GEMV_XD_PITCH * 4
+                                                          : FUSED ? gemv_fused_x_bytes<MAX_ROWS>()
+                                                                  : 16];
+    __shared__ int found_task[8];
 
     const int tid = threadIdx.x;
     int n_group = blockIdx.x % (a.n_groups * a.projections);
@@ -1234,7 +1378,11 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a
     n_group -= second ? a.n_groups : 0;
 
     int expert = 0, row_start = 0, row_end = a.rows;
-    if (a.task_count != nullptr) {
+    if constexpr (FUSED) {
+        if (a.expert_offsets != nullptr && !gemv_find_task(a, task, tid, found_task, expert, row_start, row_end)) {
+            return;
+        }
+    } else if (a.task_count != nullptr) {
         // all four loads go out together (slot `task` exists in the list's arrays whatever the count says)
         const int count = a.task_count[0];
         expert = a.task_expert[task];
@@ -1255,13 +1403,13 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a
     // touches LDS again)
     auto run = [&](int first, int nrows) {
         if (MAX_ROWS == 1 || nrows == 1) {
-            gemv_rows<TYPE, 1, FOLD>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
+            gemv_rows<TYPE, 1, FOLD, FUSED>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
         } else if (MAX_ROWS == 2 || nrows == 2) {
-            gemv_rows<TYPE, MAX_ROWS >= 2 ? 2 : 1, FOLD>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
+            gemv_rows<TYPE, MAX_ROWS >= 2 ? 2 : 1, FOLD, FUSED>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
         } else if (MAX_ROWS == 4 || nrows <= 4) {
-            gemv_rows<TYPE, MAX_ROWS >= 4 ? 4 : 1, FOLD>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
+            gemv_rows<TYPE, MAX_ROWS >= 4 ? 4 : 1, FOLD, FUSED>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
         } else {
-            gemv_rows<TYPE, MAX_ROWS >= 8 ? GEMV_ROWS : 1, FOLD>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
+            gemv_rows<TYPE, MAX_ROWS >= 8 ? GEMV_ROWS : 1, FOLD, FUSED>(a, raw, scale_lds, x_lds, grid, weights, y, n0, first, nrows, tid);
         }
     };
     if constexpr (WALK) {
@@ -1299,18 +1447,21 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_mfma_kernel(const GemvA
     }
 }
 
-template <int TYPE, int FOLD>
+static bool gemv_grouped(const GemvArgs & args) { return args.task_count != nullptr || args.expert_offsets != nullptr; }
+
+template <int TYPE, int FOLD, bool FUSED>
 static hipError_t launch_gemv_folded(const GemvArgs & args, int max_rows, unsigned grid, hipStream_t stream) {
     if (max_rows <= 1) {
-        mmq_gemv_kernel<TYPE, 1, FOLD><<<grid, GEMV_THREADS, 0, stream>>>(args);
+        mmq_gemv_kernel<TYPE, 1, FOLD, false, FUSED><<<grid, GEMV_THREADS, 0, stream>>>(args);
     } else if (max_rows <= 2) {
-        mmq_gemv_kernel<TYPE, 2, FOLD><<<grid, GEMV_THREADS, 0, stream>>>(args);
+        mmq_gemv_kernel<TYPE, 2, FOLD, false, FUSED><<<grid, GEMV_THREADS, 0, stream>>>(args);
     } else if (max_rows <= 4) {
-        mmq_gemv_kernel<TYPE, 4, FOLD><<<grid, GEMV_THREADS, 0, stream>>>(args);
-    } else if (args.task_count != nullptr || args.rows <= GEMV_ROWS) {
-        mmq_gemv_kernel<TYPE, GEMV_ROWS, FOLD><<<grid, GEMV_THREADS, 0, stream>>>(args);
-    } else if constexpr (TYPE != Q4_K && TYPE != Q5_K) {   // (dense Q4_K / Q5_K calls of that size take the matrix-core kernel)
-        mmq_gemv_kernel<TYPE, GEMV_ROWS, FOLD, true><<<grid, GEMV_THREADS, 0, stream>>>(args);
+        mmq_gemv_kernel<TYPE, 4, FOLD, false, FUSED><<<grid, GEMV_THREADS, 0, stream>>>(args);
+    } else if (gemv_grouped(args) || args.rows <= GEMV_ROWS) {
+        mmq_gemv_kernel<TYPE, GEMV_ROWS, FOLD, false, FUSED><<<grid, GEMV_THREADS, 0, stream>>>(args);
+    } else if constexpr (TYPE != Q4_K && TYPE != Q5_K && !FUSED) {
+        // (dense Q4_K / Q5_K calls of that size take the matrix-core kernel; fused dense calls are one task)
+        mmq_gemv_kernel<TYPE, GEMV_ROWS, FOLD, true, false><<<grid, GEMV_THREADS, 0, stream>>>(args);
     } else {
         return hipErrorInvalidValue;
     }
@@ -1321,7 +1472,7 @@ template <int TYPE>
 static hipError_t launch_gemv_typed(GemvArgs args, int task_slots, hipStream_t stream) {
     // no task has more rows than the call (dense: the call is the task)
     const int max_rows = args.rows < GEMV_ROWS ? args.rows : GEMV_ROWS;
-    const bool matrix_cores_only = (TYPE == Q4_K || TYPE == Q5_K) && args.task_count == nullptr && max_rows > 2;
+    const bool matrix_cores_only = (TYPE == Q4_K || TYPE == Q5_K) && !gemv_grouped(args) && max_rows > 2;
     // short K: 2 or 4 consecutive weight rows form one long row, see gemv_task
     int fold = 1;
     const int super_blocks = args.in_features / QK_K;
@@ -1340,6 +1491,9 @@ static hipError_t launch_gemv_typed(GemvArgs args, int task_slots, hipStream_t s
     const unsigned grid = static_cast<unsigned>(total);
     const ProfileScope scope(5, stream);
     if constexpr (TYPE == Q4_K || TYPE == Q5_K) {
+        if (args.x != nullptr) {
+            return hipErrorInvalidValue;   // (gemv_fuses is false for these formats)
+        }
         if (matrix_cores_only) {
             if (args.rows <= GEMV_ROWS) {
                 mmq_gemv_mfma_kernel<TYPE, GEMV_ROWS><<<grid, GEMV_THREADS, 0, stream>>>(args);
@@ -1348,34 +1502,44 @@ static hipError_t launch_gemv_typed(GemvArgs args, int task_slots, hipStream_t s
             }
             return hipGetLastError();
         }
+    } else if (args.x != nullptr) {
+        switch (fold) {
+            case 4: return launch_gemv_folded<TYPE, 4, true>(args, max_rows, grid, stream);
+            case 2: return launch_gemv_folded<TYPE, 2, true>(args, max_rows, grid, stream);
+            default: return launch_gemv_folded<TYPE, 1, true>(args, max_rows, grid, stream);
+        }
     }
     switch (fold) {
-        case 4: return launch_gemv_folded<TYPE, 4>(args, max_rows, grid, stream);
-        case 2: return launch_gemv_folded<TYPE, 2>(args, max_rows, grid, stream);
-        default: return launch_gemv_folded<TYPE, 1>(args, max_rows, grid, stream);
+        case 4: return launch_gemv_folded<TYPE, 4, false>(args, max_rows, grid, stream);
+        case 2: return launch_gemv_folded<TYPE, 2, false>(args, max_rows, grid, stream);
+        default: return launch_gemv_folded<TYPE, 1, false>(args, max_rows, grid, stream);
     }
 }
 
-hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second, int64_t bytes_per_expert,
-                           const Q8Workspace & ws, uint16_t * output, uint16_t * output_second,
-                           const TaskList * tasks, int rows, int in_features, int out_features,
-                           int quant_type, hipStream_t stream) {
-    if (!ws.by_rows()) {
-        return hipErrorInvalidValue;   // these kernels read the row-major activation layout
+static hipError_t launch_gemv_by_type(const GemvArgs & args, int task_slots, int quant_type, hipStream_t stream) {
+    switch (quant_type) {
+        case Q3_K: return launch_gemv_typed<Q3_K>(args, task_slots, stream);
+        case Q4_K: return launch_gemv_typed<Q4_K>(args, task_slots, stream);
+        case Q5_K: return launch_gemv_typed<Q5_K>(args, task_slots, stream);
+        case Q6_K: return launch_gemv_typed<Q6_K>(args, task_slots, stream);
+        case IQ2_S: return launch_gemv_typed<IQ2_S>(args, task_slots, stream);
+        default: return hipErrorInvalidValue;
     }
-    GemvArgs args;
+}
+
+// What both kinds of call share: the weights, the results, the shape.
+static GemvArgs gemv_common_args(const uint8_t * packed, const uint8_t * packed_second, int64_t bytes_per_expert,
+                                 uint16_t * output, uint16_t * output_second, int rows, int in_features,
+                                 int out_features, int quant_type) {
+    GemvArgs args = {};
     args.packed = packed;
     args.packed_second = packed_second;
+    args.y = output;
     args.y_second = output_second;
     args.projections = packed_second != nullptr ? 2 : 1;
     args.bytes_per_expert = bytes_per_expert;
     args.row_bytes = static_cast<int64_t>(in_features / QK_K) * block_bytes(quant_type);
-    args.qx = ws.q;
-    args.dx = ws.d;
-    args.sx = ws.sum;
-    args.y = output;
     args.rows = rows;
-    args.rows_padded = static_cast<int>(ws.rows_padded);
     args.in_features = in_features;
     args.out_features = out_features;
     args.n_groups = (out_features + GEMV_GN - 1) / GEMV_GN;
@@ -1385,6 +1549,47 @@ hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second
                                 (packed_second == nullptr || wide_stage_ok(packed_second, weight_bytes)) &&
                                 args.row_bytes < (1 << 24)
                             ? 1 : 0;
+    return args;
+}
+
+hipError_t launch_mmq_gemv_fused(const uint8_t * packed, const uint8_t * packed_second, int64_t bytes_per_expert,
+                                 const uint16_t * input, const int64_t * gather, int64_t input_rows,
+                                 const int64_t * expert_indices, const int32_t * expert_offsets, int num_experts,
+                                 int num_groups, uint16_t * output, uint16_t * output_second, int rows, int in_features,
+                                 int out_features, int quant_type, hipStream_t stream) {
+    if (!gemv_fuses(quant_type, rows, expert_offsets != nullptr ? num_groups : 0)) {
+        return hipErrorInvalidValue;
+    }
+    GemvArgs args = gemv_common_args(packed, packed_second, bytes_per_expert, output, output_second, rows, in_features,
+                                     out_features, quant_type);
+    args.x = input;
+    args.gather = gather;
+    args.input_rows = input_rows;
+    args.rows_padded = rows;
+    int task_slots = 1;
+    if (expert_offsets != nullptr) {
+        args.expert_indices = expert_indices;
+        args.expert_offsets = expert_offsets;
+        args.num_experts = num_experts;
+        args.num_groups = num_groups;
+        task_slots = max_tasks_for(rows, num_groups, GEMV_ROWS);
+    }
+    return launch_gemv_by_type(args, task_slots, quant_type, stream);
+}
+
+hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second, int64_t bytes_per_expert,
+                           const Q8Workspace & ws, uint16_t * output, uint16_t * output_second,
+                           const TaskList * tasks, int rows, int in_features, int out_features,
+                           int quant_type, hipStream_t stream) {
+    if (!ws.by_rows()) {
+        return hipErrorInvalidValue;   // these kernels read the row-major activation layout
+    }
+    GemvArgs args = gemv_common_args(packed, packed_second, bytes_per_expert, output, output_second, rows, in_features,
+                                     out_features, quant_type);
+    args.qx = ws.q;
+    args.dx = ws.d;
+    args.sx = ws.sum;
+    args.rows_padded = static_cast<int>(ws.rows_padded);
     int task_slots = 1;
     if (tasks != nullptr) {
         args.task_count = tasks->count;
@@ -1401,14 +1606,7 @@ hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second
         args.task_row_start = nullptr;
         args.task_row_end = nullptr;
     }
-    switch (quant_type) {
-        case Q3_K: return launch_gemv_typed<Q3_K>(args, task_slots, stream);
-        case Q4_K: return launch_gemv_typed<Q4_K>(args, task_slots, stream);
-        case Q5_K: return launch_gemv_typed<Q5_K>(args, task_slots, stream);
-        case Q6_K: return launch_gemv_typed<Q6_K>(args, task_slots, stream);
-        case IQ2_S: return launch_gemv_typed<IQ2_S>(args, task_slots, stream);
-        default: return hipErrorInvalidValue;
-    }
+    return launch_gemv_by_type(args, task_slots, quant_type, stream);
 }
 
 }  // namespace tgo

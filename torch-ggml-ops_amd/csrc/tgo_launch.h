@@ -261,6 +261,24 @@ hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second
                            const Q8Workspace & ws, uint16_t * output, uint16_t * output_second,
                            const TaskList * tasks, int rows, int in_features, int out_features,
                            int quant_type, hipStream_t stream);
+// The same from bf16 activations in one launch: every workgroup quantizes its task's rows itself and, for a grouped
+// call (`expert_offsets` set), finds its task in the group list, so neither a quantizer launch nor a task list
+// exists.  Formats whose decode-regime routines read their activations one 16-value unit per lane.
+// `gather` (or nullptr): row r of the call is row gather[r] of `input`, which has `input_rows` rows.
+// The quantization is repeated by every workgroup that shares a task's rows (one per 16 weight rows), which costs a
+// workgroup about as much as its dot products once a task has eight rows; it pays while the call is bound by its
+// launches and their latencies: dense calls of one task, grouped calls of at most 64 rows (measured on a 256-expert
+// layer: 1 token x top-8 32 -> 20 us of kernel time, 8 tokens 52 -> 48 us, 256 rows with 200 in one group 68 -> 101 us).
+constexpr int GEMV_FUSED_GROUPED_ROWS = 64;
+static inline bool gemv_fuses(int quant_type, int64_t rows, int64_t groups) {
+    const bool format = quant_type == 11 || quant_type == 14 || quant_type == 22;   // Q3_K, Q6_K, IQ2_S
+    return format && use_gemv(rows, groups) && rows <= (groups <= 0 ? GEMV_ROW_TILE : GEMV_FUSED_GROUPED_ROWS);
+}
+hipError_t launch_mmq_gemv_fused(const uint8_t * packed, const uint8_t * packed_second, int64_t bytes_per_expert,
+                                 const uint16_t * input, const int64_t * gather, int64_t input_rows,
+                                 const int64_t * expert_indices, const int32_t * expert_offsets, int num_experts,
+                                 int num_groups, uint16_t * output, uint16_t * output_second, int rows, int in_features,
+                                 int out_features, int quant_type, hipStream_t stream);
 // Cotangent in MFMA fragment order: [rows_padded/32][chunks] slabs of 1 KiB (32 rows x 16 columns), zero
 // padded; the column count is rounded up to 64 so that kernels can walk it four chunks at a time.
 static inline int cotangent_chunks(int64_t out_features) { return static_cast<int>((out_features + 63) / 64 * 4); }

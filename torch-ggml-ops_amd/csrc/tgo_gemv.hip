@@ -198,15 +198,19 @@ struct GemvUnits {
     static_assert(TOTAL < 3000, "range of the reciprocal");
 };
 template <int TYPE>
-TGO_DEVICE void gemv_stage_units(uint8_t * raw, const uint8_t * tile, int64_t row_bytes, int rows_valid, int kb0,
-                                 int chunk_blocks, int tid) {
+struct GemvUnitRegs {
+    u32x4_t unit_value[GemvUnits<TYPE>::REGS];
+    uint32_t next_value[GemvUnits<TYPE>::REGS];
+    uint32_t place[GemvUnits<TYPE>::REGS];   // LDS byte offset of the unit's first word | halfword shift << 16
+};
+// (requests the units; gemv_units_park writes them to LDS, so that a caller can put work of its own between the two)
+template <int TYPE>
+TGO_DEVICE void gemv_units_fetch(GemvUnitRegs<TYPE> & regs, const uint8_t * tile, int64_t row_bytes, int rows_valid,
+                                 int kb0, int chunk_blocks, int tid) {
     using U = GemvUnits<TYPE>;
     using W = WideStage<TYPE>;
     const uint32_t tile_m = static_cast<uint32_t>(reinterpret_cast<uintptr_t>(tile)) & 15u;
     const uint8_t * const aligned = tile - tile_m;
-    u32x4_t unit_value[U::REGS];
-    uint32_t next_value[U::REGS];
-    uint32_t place[U::REGS];   // LDS byte offset of the unit's first word | halfword shift << 16
 #pragma unroll
     for (int i = 0; i < U::REGS; ++i) {
         // ids past the pass repeat its last unit: no lane branches around a load
@@ -222,22 +226,32 @@ TGO_DEVICE void gemv_stage_units(uint8_t * raw, const uint8_t * tile, int64_t ro
         const bool carries = 16 * (unit + 1) < reach;                 // the following unit still holds bytes of the block
         const int source_unit = 16 * unit < reach ? unit : 0;         // (units past the block re-read its first one)
         const uint32_t offset = (first & ~15u) + 16u * source_unit;
-        unit_value[i] = *reinterpret_cast<const u32x4_t *>(aligned + offset);
-        next_value[i] = *reinterpret_cast<const uint32_t *>(aligned + offset + (carries ? 16u : 0u));
+        regs.unit_value[i] = *reinterpret_cast<const u32x4_t *>(aligned + offset);
+        regs.next_value[i] = *reinterpret_cast<const uint32_t *>(aligned + offset + (carries ? 16u : 0u));
         const uint32_t m = first & 15u;
         // rows and super-blocks the pass does not have are parked in their own slots (never read)
-        place[i] = static_cast<uint32_t>(slot * W::PITCH + W::FRONT + 16 * unit) - (m & 12u) + ((m & 2u) << 16);
+        regs.place[i] = static_cast<uint32_t>(slot * W::PITCH + W::FRONT + 16 * unit) - (m & 12u) + ((m & 2u) << 16);
     }
+}
+template <int TYPE>
+TGO_DEVICE void gemv_units_park(uint8_t * raw, const GemvUnitRegs<TYPE> & regs) {
 #pragma unroll
-    for (int i = 0; i < U::REGS; ++i) {
-        const uint32_t shift = place[i] >> 16;
-        const u32x4_t d = unit_value[i];
-        uint32_t * dst = reinterpret_cast<uint32_t *>(raw + (place[i] & 0xffffu));
+    for (int i = 0; i < GemvUnits<TYPE>::REGS; ++i) {
+        const uint32_t shift = regs.place[i] >> 16;
+        const u32x4_t d = regs.unit_value[i];
+        uint32_t * dst = reinterpret_cast<uint32_t *>(raw + (regs.place[i] & 0xffffu));
         dst[0] = __builtin_amdgcn_alignbyte(d.y, d.x, shift);
         dst[1] = __builtin_amdgcn_alignbyte(d.z, d.y, shift);
         dst[2] = __builtin_amdgcn_alignbyte(d.w, d.z, shift);
-        dst[3] = __builtin_amdgcn_alignbyte(next_value[i], d.w, shift);
+        dst[3] = __builtin_amdgcn_alignbyte(regs.next_value[i], d.w, shift);
     }
+}
+template <int TYPE>
+TGO_DEVICE void gemv_stage_units(uint8_t * raw, const uint8_t * tile, int64_t row_bytes, int rows_valid, int kb0,
+                                 int chunk_blocks, int tid) {
+    GemvUnitRegs<TYPE> regs;
+    gemv_units_fetch<TYPE>(regs, tile, row_bytes, rows_valid, kb0, chunk_blocks, tid);
+    gemv_units_park<TYPE>(raw, regs);
 }
 
 // Register-staged copy for the formats whose blocks are whole 16-byte units: the loads of a pass are issued into
@@ -515,17 +529,7 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, uint8_t * x_lds, co
             }
         }
         __syncthreads();   // the previous pass is done with `raw` (and with the activations in LDS)
-        if (unit_staging) {
-            gemv_stage_units<TYPE>(raw, weights + static_cast<int64_t>(n0) * long_row_bytes, long_row_bytes,
-                                   min(GEMV_GN, long_rows - n0), kb0, chunk_blocks, tid);
-        } else if ((long_row_bytes & 15) == 0) {
-            gemv_stage_pieces<TYPE, 16>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
-        } else if ((long_row_bytes & 3) == 0) {
-            gemv_stage_pieces<TYPE, 4>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
-        } else {
-            gemv_stage<TYPE>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
-        }
-        if constexpr (FUSED) {
+        const auto quantize_rows = [&]() __attribute__((always_inline)) {
             if (x_mine) {
 #pragma unroll
                 for (int r = 0; r < ROWS; ++r) {
@@ -544,6 +548,27 @@ TGO_DEVICE void gemv_task(const GemvArgs & a, uint8_t * raw, uint8_t * x_lds, co
                         xd_lds[r * GEMV_CHUNK * 8 + (tid >> 2)] = d;
                     }
                 }
+            }
+        };
+        if (unit_staging) {
+            // (the activations were requested first and are quantized while the weights travel)
+            GemvUnitRegs<TYPE> units;
+            gemv_units_fetch<TYPE>(units, weights + static_cast<int64_t>(n0) * long_row_bytes, long_row_bytes,
+                                   min(GEMV_GN, long_rows - n0), kb0, chunk_blocks, tid);
+            if constexpr (FUSED) {
+                quantize_rows();
+            }
+            gemv_units_park<TYPE>(raw, units);
+        } else if ((long_row_bytes & 15) == 0) {
+            gemv_stage_pieces<TYPE, 16>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
+        } else if ((long_row_bytes & 3) == 0) {
+            gemv_stage_pieces<TYPE, 4>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
+        } else {
+            gemv_stage<TYPE>(raw, weights, long_row_bytes, n0, long_rows, kb0, chunk_blocks, tid);
+        }
+        if constexpr (FUSED) {
+            if (!unit_staging) {
+                quantize_rows();
             }
         }
         __syncthreads();

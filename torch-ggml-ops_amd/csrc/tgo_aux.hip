@@ -113,6 +113,12 @@ __global__ __launch_bounds__(256) void quantize_q8_1_rows_kernel(const uint16_t 
     }
 }
 
+// Where 16-byte piece `piece` of a quantizer's LDS tile lives.  The lanes of a store differ in the 8 values of K they
+// hold, and those land a whole run of 32 pieces (512 bytes) apart: all on the same four banks.  So a piece's place inside
+// its run is exchanged by the run's number, which spreads the pieces of one store over all banks; the copy out of the
+// tile reads the pieces back through the same exchange.
+TGO_DEVICE int swizzled_piece(int piece) { return piece ^ ((piece >> 5) & 15); }
+
 // LAYOUT_HALF_TILES: the quants leave as fp16 numbers for the fp16-operand forward kernels, 16 KiB per workgroup:
 // per 32-value block two 1 KiB slabs (k-halves of 16 values), each 64 pieces of eight values = (eighth of the
 // k-half, row).
@@ -184,11 +190,12 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
         quantize_eight(row_bits, x, packed, d, total, halves, magnitude);
         const int half = quarter >> 1;
         if constexpr (WIDE_VALUES) {
-            // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
-            *reinterpret_cast<uint4 *>(tile + block * 2048 + half * 1024 + (rr + 32 * (quarter & 1)) * 16) =
+            // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2, i.e. piece lane_k * 32 + rr
+            *reinterpret_cast<uint4 *>(tile + swizzled_piece(lane_k * 32 + rr) * 16) =
                 make_uint4(halves[0], halves[1], halves[2], halves[3]);
         } else {
-            uint2 * dst = reinterpret_cast<uint2 *>(tile + block * 1024 + (rr + 32 * half) * 16 + 8 * (quarter & 1));
+            // (piece (2 * block + half) * 32 + rr, one half of it per lane)
+            uint2 * dst = reinterpret_cast<uint2 *>(tile + swizzled_piece((lane_k >> 1) * 32 + rr) * 16 + 8 * (quarter & 1));
             *dst = make_uint2(packed[0], packed[1]);
         }
         if (quarter == 0) {
@@ -210,7 +217,7 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const uint16_t * __r
     const uint4 * src = reinterpret_cast<const uint4 *>(tile);
 #pragma unroll
     for (int piece = 0; piece < 8 * BLOCK_BYTES / 16 / 256; ++piece) {
-        dst[tid + 256 * piece] = src[tid + 256 * piece];
+        dst[tid + 256 * piece] = src[swizzled_piece(tid + 256 * piece)];
     }
 }
 
@@ -300,8 +307,8 @@ __global__ __launch_bounds__(256) void quantize_q8_1_scaled_kernel(const uint16_
                                     static_cast<_Float16>(static_cast<float>(magnitude[2 * pair + 1]) * lane_scale)};
             halves[pair] = __builtin_bit_cast(uint32_t, values) | (words[pair] & 0x80008000u);
         }
-        // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2
-        *reinterpret_cast<uint4 *>(tile + block * 2048 + (quarter >> 1) * 1024 + (rr + 32 * (quarter & 1)) * 16) =
+        // values 8 * quarter .. + 7 of the block: k-half quarter / 2, eighth quarter % 2, i.e. piece lane_k * 32 + rr
+        *reinterpret_cast<uint4 *>(tile + swizzled_piece(lane_k * 32 + rr) * 16) =
             make_uint4(halves[0], halves[1], halves[2], halves[3]);
         if (quarter == 0) {
             scales[0][block][rr] = d;
@@ -332,7 +339,7 @@ __global__ __launch_bounds__(256) void quantize_q8_1_scaled_kernel(const uint16_
     const uint4 * src = reinterpret_cast<const uint4 *>(tile);
 #pragma unroll
     for (int piece = 0; piece < 4; ++piece) {
-        dst[tid + 256 * piece] = src[tid + 256 * piece];
+        dst[tid + 256 * piece] = src[swizzled_piece(tid + 256 * piece)];
     }
 }
 

@@ -196,6 +196,28 @@ int tgo_grouped_mmq_swiglu(const void * input_bf16, const int64_t * row_index, i
                            int64_t in_features, int64_t out_features, int64_t num_experts,
                            int64_t num_groups, int quant_type, void * stream);
 
+/* The cotangent of tgo_grouped_mmq_swiglu's activated output taken back to the two projections, elementwise over
+ * `count` bf16 values: with s = sigmoid(gate),
+ *   d_up = bf16(grad_activated * gate * s),   d_gate = bf16(grad_activated * up * s * (1 + gate * (1 - s)) + grad_gate),
+ * every factor read as bf16, the arithmetic in fp32.  `grad_gate_bf16` (a cotangent of the gate output itself) may be
+ * NULL.  d_gate and d_up are what tgo_grouped_mmq_grad_input takes as its two cotangents.  No counterpart in the
+ * reference, whose pair operator leaves the activation and its derivative to the caller's tensor operations
+ * (csrc/mmq_hip.cu:1054-1193). */
+int tgo_swiglu_backward(const void * gate_bf16, const void * up_bf16, const void * grad_activated_bf16,
+                        const void * grad_gate_bf16, void * d_gate_bf16, void * d_up_bf16, int64_t count, void * stream);
+
+/* The row gather of the gathered entry points run backwards: the gradients of the sorted rows summed per token,
+ *   output[t, :] = bf16( sum of rows[order[i], :] for starts[t] <= i < starts[t + 1] )      (t < tokens)
+ * rows bf16 [num_rows, features]; order int64 [num_rows] lists the sorted rows token by token (a stable sort of the
+ * gather index: rows of one token stay in row order); starts int64 [tokens + 1] is where each token's run begins.  The
+ * rows of a run are added in list order in fp32 and rounded once: no atomics, the same bits on every run.  Entries of
+ * `order` outside [0, num_rows) and the parts of a run outside the list contribute nothing, so rows whose gather index
+ * named no token are left out by ending the last run before them.  `features` is a multiple of 8.  No counterpart in
+ * the reference, whose operators take expert-sorted rows and leave gather and scatter to the caller
+ * (torch_ggml_ops/grouped_mmq.py:216). */
+int tgo_rows_to_tokens(const void * rows_bf16, const int64_t * order, const int64_t * starts, void * output_bf16,
+                       int64_t tokens, int64_t num_rows, int64_t features, void * stream);
+
 /* Routing-weighted return from expert-sorted rows to tokens:
  *   output[t, :] = sum_j slot_weights[t, j] * rows[slot_rows[t, j], :]      (t < tokens, j < top_k)
  * rows bf16 [num_rows, features], slot_rows int64 [tokens, top_k] (the sorted row of each choice; a value

@@ -184,17 +184,24 @@ def test_synthetic_generators_are_seeded_and_well_formed(package, oracle):
     assert (indices[1:] > indices[:-1]).all() and (offsets[1:] > offsets[:-1]).all()
 
 
-def test_token_scatter_masks_rows_outside_the_input(package):
-    """The per-token sum behind the gathered operators' gradients, on the CPU: rows whose index lies outside the
-    token range are dropped (no out-of-range index is ever used), the others add up per token in fp32."""
-    from torch_ggml_ops.gathered import _scatter_to_tokens
+def test_token_runs_drop_rows_outside_the_input(package):
+    """The host half of the per-token sum behind the gathered operators' gradients: the rows listed token by token in
+    row order, with the rows whose index lies outside the token range behind the last run (the kernel that adds the
+    runs up never sees them).  Summing the runs on the CPU gives the per-token sums."""
+    from torch_ggml_ops.gathered import _token_runs
 
     grad_rows = torch.arange(24, dtype=torch.float32).reshape(6, 4).to(torch.bfloat16)
     row_index = torch.tensor([2, -1, 0, 9, 3, 2])
-    result = _scatter_to_tokens(grad_rows, row_index, 4)
+    order, starts = _token_runs(row_index, 4)
+    assert order.dtype == torch.int64 and starts.dtype == torch.int64
+    assert starts.tolist() == [0, 1, 1, 3, 4]
+    assert order.tolist()[:4] == [2, 0, 5, 4] and sorted(order.tolist()[4:]) == [1, 3]
+    result = torch.zeros(4, 4)
+    for token in range(4):
+        for row in order[starts[token]:starts[token + 1]].tolist():
+            result[token] += grad_rows[row].float()
     expected = torch.zeros(4, 4)
     for row, token in enumerate(row_index.tolist()):
         if 0 <= token < 4:
             expected[token] += grad_rows[row].float()
-    assert result.dtype == torch.bfloat16
-    torch.testing.assert_close(result.float(), expected.to(torch.bfloat16).float(), rtol=0, atol=0)
+    torch.testing.assert_close(result, expected, rtol=0, atol=0)

@@ -146,3 +146,23 @@ def test_gathered_rejects_bad_index(ops):
         tgo.grouped_mmq_gathered(hidden, torch.arange(4, device="cuda", dtype=torch.int32), weight, indices, offsets, 12, 32)
     with pytest.raises(RuntimeError, match="one-dimensional"):
         tgo.grouped_mmq_gathered(hidden, torch.zeros((2, 2), device="cuda", dtype=torch.int64), weight, indices, offsets, 12, 32)
+
+
+@pytest.mark.parametrize("tokens,rows,features", ((5, 23, 256), (97, 388, 2048), (300, 64, 2304)))
+def test_rows_to_tokens_kernel_equals_an_ordered_index_put(ops, tokens, rows, features):
+    """The scatter of the gathered operators' backward (tgo_rows_to_tokens over a stable sort of the gather index)
+    against index_put_(accumulate=True) on fp32 copies, which also adds each token's rows in row order: the same bits.
+    Some rows name no token (dropped), some tokens have no row (zeros)."""
+    from torch_ggml_ops import gathered
+
+    generator = torch.Generator(device="cuda").manual_seed(tokens + rows)
+    grad_rows = torch.randn(rows, features, device="cuda", generator=generator).to(torch.bfloat16)
+    row_index = torch.randint(0, tokens, (rows,), device="cuda", generator=generator)
+    row_index[::7] = -1
+    row_index[3::11] = tokens + 5
+    actual = gathered._scatter_to_tokens(grad_rows, row_index, tokens)
+    present = (row_index >= 0) & (row_index < tokens)
+    total = torch.zeros((tokens, features), dtype=torch.float32, device="cuda")
+    total.index_put_((row_index.clamp(0, tokens - 1),), grad_rows.float() * present.unsqueeze(1), accumulate=True)
+    assert actual.shape == (tokens, features) and actual.dtype == torch.bfloat16
+    torch.testing.assert_close(actual, total.to(torch.bfloat16), rtol=0, atol=0)

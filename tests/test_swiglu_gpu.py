@@ -152,3 +152,32 @@ def test_gradient_matches_the_unfused_chain(ops, gathered):
     assert fused_in.grad.shape == plain_in.grad.shape
     # both chains round d_gate and d_up to bf16 before the grad-input kernel, at slightly different points
     assert nrmse(f32(fused_in.grad), f32(plain_in.grad)) < 1e-2
+
+
+@pytest.mark.parametrize("count", (8 * 1000, 4099))
+@pytest.mark.parametrize("direct", (False, True))
+def test_activation_backward_kernel_matches_the_formulas(ops, count, direct):
+    """tgo_swiglu_backward against the same formulas written with fp32 tensor operations: d_up = dy * gate * s and
+    d_gate = dy * up * s * (1 + gate * (1 - s)) (+ a cotangent of the gate itself), rounded to bf16 once.  The kernel's
+    sigmoid uses the hardware's exponential and reciprocal, so a result may land on the neighbouring bf16 value: the
+    bound is one bf16 step (2^-7 relative), and large gates of either sign must stay finite."""
+    from torch_ggml_ops import swiglu as module
+
+    generator = torch.Generator(device="cuda").manual_seed(count)
+    gate = (4.0 * torch.randn(count, device="cuda", generator=generator)).to(torch.bfloat16)
+    gate[:6] = torch.tensor([0.0, -0.0, 60.0, -60.0, 200.0, -200.0], dtype=torch.bfloat16)
+    up = torch.randn(count, device="cuda", generator=generator).to(torch.bfloat16)
+    dy = torch.randn(count, device="cuda", generator=generator).to(torch.bfloat16)
+    grad_gate = torch.randn(count, device="cuda", generator=generator).to(torch.bfloat16) if direct else None
+    if count % 8:   # an odd length and a start off the 16-byte grid: the element-at-a-time path
+        gate, up, dy = gate[1:], up[1:], dy[1:]
+        grad_gate = None if grad_gate is None else grad_gate[1:]
+    d_gate, d_up = module._activation_backward(gate, up, dy, grad_gate)
+    g, u, y = gate.float(), up.float(), dy.float()
+    s = torch.sigmoid(g)
+    expected_up = y * (g * s)
+    expected_gate = y * u * (s * (1.0 + g * (1.0 - s))) + (0.0 if grad_gate is None else grad_gate.float())
+    assert torch.isfinite(d_gate).all() and torch.isfinite(d_up).all()
+    for actual, expected in ((d_up, expected_up), (d_gate, expected_gate)):
+        error = (actual.float() - expected).abs()
+        assert bool((error <= 2.0**-7 * expected.abs() + 1e-30).all()), float((error / expected.abs().clamp_min(1e-30)).max())

@@ -190,7 +190,7 @@ ProfileScope::~ProfileScope() {
 
 extern "C" {
 
-int tgo_version(void) { return 111; }
+int tgo_version(void) { return 112; }
 
 int tgo_profile_enable(int enabled) {
     std::lock_guard<std::mutex> lock(g_profile_mutex);
@@ -536,6 +536,23 @@ int tgo_grouped_mmq_swiglu(const void * input_bf16, const int64_t * row_index, i
                            num_groups, quant_type, stream, true);
 }
 
+int tgo_swiglu_backward(const void * gate_bf16, const void * up_bf16, const void * grad_activated_bf16,
+                        const void * grad_gate_bf16, void * d_gate_bf16, void * d_up_bf16, int64_t count, void * stream) {
+    if (count <= 0) {
+        return fail(TGO_ERR_INVALID, "count must be positive; got %lld", static_cast<long long>(count));
+    }
+    if (gate_bf16 == nullptr || up_bf16 == nullptr || grad_activated_bf16 == nullptr || d_gate_bf16 == nullptr ||
+        d_up_bf16 == nullptr) {
+        return fail(TGO_ERR_INVALID, "gate, up, grad_activated, d_gate and d_up must not be null");
+    }
+    return check_hip(tgo::launch_swiglu_backward_rows(
+                         static_cast<const uint16_t *>(gate_bf16), static_cast<const uint16_t *>(up_bf16),
+                         static_cast<const uint16_t *>(grad_activated_bf16), static_cast<const uint16_t *>(grad_gate_bf16),
+                         static_cast<uint16_t *>(d_gate_bf16), static_cast<uint16_t *>(d_up_bf16), count,
+                         static_cast<hipStream_t>(stream)),
+                     "swiglu_backward launch");
+}
+
 int tgo_moe_combine(const void * rows_bf16, const int64_t * slot_rows, const float * slot_weights,
                     void * output_bf16, int64_t tokens, int64_t top_k, int64_t num_rows, int64_t features,
                     void * stream) {
@@ -560,6 +577,29 @@ int tgo_moe_combine(const void * rows_bf16, const int64_t * slot_rows, const flo
                                              static_cast<int>(top_k), num_rows, static_cast<int>(features),
                                              static_cast<hipStream_t>(stream)),
                      "moe_combine launch");
+}
+
+int tgo_rows_to_tokens(const void * rows_bf16, const int64_t * order, const int64_t * starts, void * output_bf16,
+                       int64_t tokens, int64_t num_rows, int64_t features, void * stream) {
+    if (tokens <= 0 || num_rows <= 0) {
+        return fail(TGO_ERR_INVALID, "tokens and num_rows must be positive");
+    }
+    if (features <= 0 || features % 8 != 0) {
+        return fail(TGO_ERR_INVALID, "features must be a positive multiple of 8; got %lld",
+                    static_cast<long long>(features));
+    }
+    if (tokens > INT_LIMIT || features > INT_LIMIT || num_rows > INT_LIMIT || (features + 2047) / 2048 > 65535) {
+        return fail(TGO_ERR_INVALID, "a dimension exceeds the kernel limit");
+    }
+    TGO_TRY(check_pointer(rows_bf16, "rows"));
+    TGO_TRY(check_pointer(output_bf16, "output"));
+    if (order == nullptr || starts == nullptr) {
+        return fail(TGO_ERR_INVALID, "order and starts must not be null");
+    }
+    return check_hip(tgo::launch_rows_to_tokens(static_cast<const uint16_t *>(rows_bf16), order, starts,
+                                                static_cast<uint16_t *>(output_bf16), static_cast<int>(tokens), num_rows,
+                                                static_cast<int>(features), static_cast<hipStream_t>(stream)),
+                     "rows_to_tokens launch");
 }
 
 // Shared body of the grouped grad-input entry points; `row_token` is null for a cotangent given row by row.

@@ -564,6 +564,115 @@ hipError_t launch_swiglu_rows(const uint16_t * gate, uint16_t * up_then_activate
     return hipGetLastError();
 }
 
+// The gather of the grouped operators run backwards: out[t, :] = bf16(sum of rows[order[i], :] for i in
+// [starts[t], starts[t + 1])), added in list order in fp32 and rounded once (no atomics: the same bits every time).
+// `order` lists the sorted rows token by token, `starts` where each token's run begins.  Entries that name no row,
+// and runs that reach outside the list, contribute nothing.  Same shape of work as moe_combine_kernel.
+__global__ __launch_bounds__(256) void rows_to_tokens_kernel(const uint16_t * __restrict__ rows,
+                                                             const int64_t * __restrict__ order,
+                                                             const int64_t * __restrict__ starts,
+                                                             uint16_t * __restrict__ out, int64_t num_rows, int features) {
+    const int64_t token = blockIdx.x;
+    const int feature = blockIdx.y * COMBINE_SPAN + threadIdx.x * 8;
+    if (feature >= features) {
+        return;
+    }
+    const int64_t begin = max(starts[token], int64_t{0});
+    const int64_t end = min(starts[token + 1], num_rows);
+    float acc[8] = {};
+    for (int64_t first = begin; first < end; first += 4) {
+        uint4 bits[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t row = order[min(first + u, end - 1)];
+            const bool present = first + u < end && row >= 0 && row < num_rows;
+            bits[u] = present ? *reinterpret_cast<const uint4 *>(rows + row * features + feature) : uint4{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const uint32_t words[4] = {bits[u].x, bits[u].y, bits[u].z, bits[u].w};
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                acc[2 * i] += bf16_bits_to_float(words[i] & 0xffffu);
+                acc[2 * i + 1] += bf16_bits_to_float(words[i] >> 16);
+            }
+        }
+    }
+    *reinterpret_cast<uint4 *>(out + token * features + feature) =
+        uint4{pack_bf16x2(acc[0], acc[1]), pack_bf16x2(acc[2], acc[3]), pack_bf16x2(acc[4], acc[5]), pack_bf16x2(acc[6], acc[7])};
+}
+
+hipError_t launch_rows_to_tokens(const uint16_t * rows, const int64_t * order, const int64_t * starts, uint16_t * out,
+                                 int tokens, int64_t num_rows, int features, hipStream_t stream) {
+    const dim3 grid(static_cast<unsigned>(tokens), static_cast<unsigned>((features + COMBINE_SPAN - 1) / COMBINE_SPAN));
+    const ProfileScope scope(7, stream);
+    rows_to_tokens_kernel<<<grid, 256, 0, stream>>>(rows, order, starts, out, num_rows, features);
+    return hipGetLastError();
+}
+
+// The activation's cotangent taken back to the two projections, elementwise: with s = sigmoid(gate),
+//   d_up = bf16(dy * gate * s),   d_gate = bf16(dy * up * s * (1 + gate * (1 - s)) [+ grad_gate]),
+// all factors read as bf16 and multiplied in fp32.  `grad_gate` (a cotangent that reached the gate output itself) may
+// be null.  One pass over five (six) tensors instead of the dozen fp32 passes of the same formulas written with
+// tensor operations.
+TGO_DEVICE void swiglu_backward(float gate, float up, float dy, float direct, float & d_gate, float & d_up) {
+    const float s = __builtin_amdgcn_rcpf(1.0f + __expf(-gate));
+    d_up = dy * (gate * s);
+    d_gate = dy * up * (s * (1.0f + gate * (1.0f - s))) + direct;
+}
+
+__global__ __launch_bounds__(256) void swiglu_backward_rows_kernel(const uint16_t * __restrict__ gate,
+                                                                    const uint16_t * __restrict__ up,
+                                                                    const uint16_t * __restrict__ grad_activated,
+                                                                    const uint16_t * __restrict__ grad_gate,
+                                                                    uint16_t * __restrict__ d_gate,
+                                                                    uint16_t * __restrict__ d_up, int64_t count, int vector) {
+    const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
+    const int64_t first = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
+    const int64_t pieces = vector != 0 ? count / 8 : 0;
+    for (int64_t piece = first; piece < pieces; piece += stride) {
+        const uint4 g4 = reinterpret_cast<const uint4 *>(gate)[piece];
+        const uint4 u4 = reinterpret_cast<const uint4 *>(up)[piece];
+        const uint4 y4 = reinterpret_cast<const uint4 *>(grad_activated)[piece];
+        const uint4 r4 = grad_gate != nullptr ? reinterpret_cast<const uint4 *>(grad_gate)[piece] : uint4{0, 0, 0, 0};
+        const uint32_t g[4] = {g4.x, g4.y, g4.z, g4.w}, u[4] = {u4.x, u4.y, u4.z, u4.w};
+        const uint32_t y[4] = {y4.x, y4.y, y4.z, y4.w}, r[4] = {r4.x, r4.y, r4.z, r4.w};
+        uint32_t out_gate[4], out_up[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float dg[2], du[2];
+            swiglu_backward(bf16_bits_to_float(g[i] & 0xffffu), bf16_bits_to_float(u[i] & 0xffffu),
+                            bf16_bits_to_float(y[i] & 0xffffu), bf16_bits_to_float(r[i] & 0xffffu), dg[0], du[0]);
+            swiglu_backward(bf16_bits_to_float(g[i] >> 16), bf16_bits_to_float(u[i] >> 16), bf16_bits_to_float(y[i] >> 16),
+                            bf16_bits_to_float(r[i] >> 16), dg[1], du[1]);
+            out_gate[i] = pack_bf16x2(dg[0], dg[1]);
+            out_up[i] = pack_bf16x2(du[0], du[1]);
+        }
+        reinterpret_cast<uint4 *>(d_gate)[piece] = uint4{out_gate[0], out_gate[1], out_gate[2], out_gate[3]};
+        reinterpret_cast<uint4 *>(d_up)[piece] = uint4{out_up[0], out_up[1], out_up[2], out_up[3]};
+    }
+    for (int64_t index = pieces * 8 + first; index < count; index += stride) {
+        float dg, du;
+        swiglu_backward(bf16_bits_to_float(gate[index]), bf16_bits_to_float(up[index]), bf16_bits_to_float(grad_activated[index]),
+                        grad_gate != nullptr ? bf16_bits_to_float(grad_gate[index]) : 0.0f, dg, du);
+        d_gate[index] = to_bf16_bits(dg);
+        d_up[index] = to_bf16_bits(du);
+    }
+}
+
+hipError_t launch_swiglu_backward_rows(const uint16_t * gate, const uint16_t * up, const uint16_t * grad_activated,
+                                       const uint16_t * grad_gate, uint16_t * d_gate, uint16_t * d_up, int64_t count,
+                                       hipStream_t stream) {
+    const uintptr_t addresses = reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) |
+                                reinterpret_cast<uintptr_t>(grad_activated) | reinterpret_cast<uintptr_t>(grad_gate) |
+                                reinterpret_cast<uintptr_t>(d_gate) | reinterpret_cast<uintptr_t>(d_up);
+    const int vector = addresses % 16 == 0;
+    const int64_t blocks = (count / (vector != 0 ? 8 : 1) + 255) / 256;
+    swiglu_backward_rows_kernel<<<static_cast<unsigned>(blocks < 1 ? 1 : blocks > 8 * 256 * 8 ? 8 * 256 * 8 : blocks), 256, 0,
+                                  stream>>>(gate, up, grad_activated, grad_gate, d_gate, d_up, count, vector);
+    return hipGetLastError();
+}
+
 hipError_t launch_moe_combine(const uint16_t * rows, const int64_t * slot_rows, const float * slot_weights,
                               uint16_t * out, int tokens, int top_k, int64_t num_rows, int features,
                               hipStream_t stream) {

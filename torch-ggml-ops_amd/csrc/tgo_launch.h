@@ -235,6 +235,14 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
                                 int64_t input_rows = 0, const TaskBuild * build = nullptr);
 // up_then_activated[i] = swiglu(gate[i], up_then_activated[i]) over `count` bf16 values (timed with the forward kernels).
 hipError_t launch_swiglu_rows(const uint16_t * gate, uint16_t * up_then_activated, int64_t count, hipStream_t stream);
+// out[t, :] = sum of rows[order[i], :] over i in [starts[t], starts[t + 1]), in list order (fp32, one rounding).
+hipError_t launch_rows_to_tokens(const uint16_t * rows, const int64_t * order, const int64_t * starts, uint16_t * out,
+                                 int tokens, int64_t num_rows, int features, hipStream_t stream);
+// d_gate, d_up of silu(gate) * up for the cotangent `grad_activated` (and `grad_gate`, a cotangent of the gate output
+// itself, or nullptr), elementwise over `count` bf16 values.
+hipError_t launch_swiglu_backward_rows(const uint16_t * gate, const uint16_t * up, const uint16_t * grad_activated,
+                                       const uint16_t * grad_gate, uint16_t * d_gate, uint16_t * d_up, int64_t count,
+                                       hipStream_t stream);
 // Turns `count` bf16 outputs into NaN when the workspace's tag is not the layout of `ws` (runs behind the multiply kernel).
 hipError_t launch_workspace_guard(const Q8Workspace & ws, uint16_t * out, int64_t count, hipStream_t stream);
 hipError_t launch_q8_unpack(const Q8Workspace & ws, int8_t * q, float * d, float * sum, int64_t rows,

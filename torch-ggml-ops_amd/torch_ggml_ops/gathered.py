@@ -17,6 +17,7 @@ from __future__ import annotations
 
 import torch
 
+from . import _native
 from .grouped_mmq import _forward as _grouped_forward
 from .grouped_mmq import _grad_input as _grouped_grad_input
 
@@ -70,20 +71,35 @@ def _rows_grad_input(first_grad, second_grad, first_weight, second_weight, exper
     )
 
 
-def _scatter_to_tokens(grad_rows: torch.Tensor, row_index: torch.Tensor, tokens: int) -> torch.Tensor:
-    """Sum of the sorted rows' gradients per token: fp32 accumulation, one rounding to bf16.
-
-    Rows whose index lies outside ``[0, tokens)`` were zeros in the forward and are dropped here (the index
-    is clamped and the row masked, so no out-of-range index reaches the device).  The sum runs through
-    ``index_put_(accumulate=True)``, which sorts the indices and adds each token's rows in row order: the
-    result does not depend on scheduling, unlike the atomic adds of ``index_add_``.
-    """
+def _token_runs(row_index: torch.Tensor, tokens: int):
+    """The sorted rows listed token by token: ``order[starts[t]:starts[t + 1]]`` are the rows of token ``t`` in row
+    order.  Rows whose index names no token sort behind the last run (``starts[tokens]`` ends before them)."""
     present = (row_index >= 0) & (row_index < tokens)
-    safe = row_index.clamp(0, tokens - 1)
-    values = grad_rows.float() * present.unsqueeze(1)
-    total = torch.zeros((tokens, grad_rows.shape[1]), dtype=torch.float32, device=grad_rows.device)
-    total.index_put_((safe,), values, accumulate=True)
-    return total.to(grad_rows.dtype)
+    key = torch.where(present, row_index, tokens)
+    sorted_key, order = torch.sort(key, stable=True)
+    starts = torch.searchsorted(sorted_key, torch.arange(tokens + 1, device=key.device, dtype=key.dtype))
+    return order, starts
+
+
+def _scatter_to_tokens(grad_rows: torch.Tensor, row_index: torch.Tensor, tokens: int) -> torch.Tensor:
+    """Sum of the sorted rows' gradients per token: fp32 accumulation in row order, one rounding to bf16.
+
+    Rows whose index lies outside ``[0, tokens)`` were zeros in the forward and are dropped here.  The rows are
+    listed token by token with a stable sort of the index (absent rows sort behind the last token), and one kernel
+    adds each token's rows in that order (``tgo_rows_to_tokens``): no atomics, so the result does not depend on
+    scheduling, and no data-dependent shapes, so the backward can be captured in a graph.
+    """
+    grad_rows = grad_rows.contiguous()
+    order, starts = _token_runs(row_index, tokens)
+    out = torch.empty((tokens, grad_rows.shape[1]), dtype=grad_rows.dtype, device=grad_rows.device)
+    with torch.cuda.device(grad_rows.device):
+        _native.check(
+            _native.lib.tgo_rows_to_tokens(
+                grad_rows.data_ptr(), order.data_ptr(), starts.data_ptr(), out.data_ptr(), tokens, grad_rows.shape[0],
+                grad_rows.shape[1], torch.cuda.current_stream(grad_rows.device).cuda_stream,
+            )
+        )
+    return out
 
 
 def _setup_gathered_context(ctx, inputs, output) -> None:

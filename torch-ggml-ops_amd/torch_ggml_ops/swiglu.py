@@ -9,8 +9,8 @@ once.  The reference has no such operator (its pair operator ends at the two pro
 csrc/mmq_hip.cu:1054-1193).
 
 The gradient with respect to the input recomputes the up projection (one grouped forward) instead
-of keeping it: the gate is saved, ``d_gate`` and ``d_up`` follow elementwise, and the fused pair
-grad-input finishes.
+of keeping it: the gate is saved, ``d_gate`` and ``d_up`` follow from one elementwise kernel
+(``tgo_swiglu_backward``), and the fused pair grad-input finishes.
 """
 
 from __future__ import annotations
@@ -19,6 +19,7 @@ from typing import Optional
 
 import torch
 
+from . import _native
 from .grouped_mmq import _forward as _grouped_forward
 from .gathered import _rows_grad_input, _scatter_to_tokens
 
@@ -48,6 +49,22 @@ def _swiglu_fake(
     return input.new_empty((rows, out_features)), input.new_empty((rows, out_features))
 
 
+def _activation_backward(gate, up, grad_activated, grad_gate):
+    """(d_gate, d_up) of ``silu(gate) * up`` for the cotangent ``grad_activated`` (plus ``grad_gate``, a cotangent of
+    the gate output itself, or None): one elementwise kernel, bf16 in and out, fp32 arithmetic."""
+    tensors = [gate, up, grad_activated] + ([] if grad_gate is None else [grad_gate])
+    gate, up, grad_activated, *rest = [t.contiguous() for t in tensors]
+    d_gate, d_up = torch.empty_like(gate), torch.empty_like(gate)
+    with torch.cuda.device(gate.device):
+        _native.check(
+            _native.lib.tgo_swiglu_backward(
+                gate.data_ptr(), up.data_ptr(), grad_activated.data_ptr(), rest[0].data_ptr() if rest else None,
+                d_gate.data_ptr(), d_up.data_ptr(), gate.numel(), torch.cuda.current_stream(gate.device).cuda_stream,
+            )
+        )
+    return d_gate, d_up
+
+
 def _setup_context(ctx, inputs, output) -> None:
     input, row_index, gate_weight, up_weight, expert_indices, expert_offsets, quant_type, out_features = inputs
     ctx.quant_type, ctx.out_features = quant_type, out_features
@@ -61,18 +78,13 @@ def _backward(ctx, grad_activated, grad_gate):
     grad_input = None
     if ctx.needs_input_grad[0] and (grad_activated is not None or grad_gate is not None):
         input, row_index, gate_weight, up_weight, expert_indices, expert_offsets, gate = ctx.saved_tensors
-        d_gate = None if grad_gate is None else grad_gate.float()
+        d_gate = grad_gate
         d_up = None
         if grad_activated is not None:
             up = _grouped_forward(
                 input, up_weight, None, expert_indices, expert_offsets, ctx.quant_type, ctx.out_features, row_index
             )[0]
-            g, dy = gate.float(), grad_activated.float()
-            sigmoid = torch.sigmoid(g)
-            d_up = (dy * (g * sigmoid)).to(gate.dtype)
-            through = dy * up.float() * (sigmoid * (1.0 + g * (1.0 - sigmoid)))
-            d_gate = through if d_gate is None else d_gate + through
-        d_gate = d_gate.to(gate.dtype)
+            d_gate, d_up = _activation_backward(gate, up, grad_activated, grad_gate)
         if d_up is not None:
             grad_rows = _rows_grad_input(
                 d_gate, d_up, gate_weight, up_weight, expert_indices, expert_offsets, ctx.quant_type, ctx.in_features

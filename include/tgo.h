@@ -196,6 +196,12 @@ int tgo_grouped_mmq_swiglu(const void * input_bf16, const int64_t * row_index, i
                            int64_t in_features, int64_t out_features, int64_t num_experts,
                            int64_t num_groups, int quant_type, void * stream);
 
+/* activated[i] = bf16( silu(gate[i]) * up[i] ) over `count` bf16 values, fp32 arithmetic: the elementwise pass that
+ * tgo_grouped_mmq_swiglu runs itself after a scaled-operand pair, for a caller that ran the pair (tgo_grouped_mmq_forward)
+ * and wants to keep the up projection, e.g. for the backward pass.  `activated_bf16` may be `up_bf16`.  No counterpart in
+ * the reference (the activation is the caller's tensor operation there, csrc/mmq_hip.cu:1054-1193). */
+int tgo_swiglu_rows(const void * gate_bf16, const void * up_bf16, void * activated_bf16, int64_t count, void * stream);
+
 /* The cotangent of tgo_grouped_mmq_swiglu's activated output taken back to the two projections, elementwise over
  * `count` bf16 values: with s = sigmoid(gate),
  *   d_up = bf16(grad_activated * gate * s),   d_gate = bf16(grad_activated * up * s * (1 + gate * (1 - s)) + grad_gate),

@@ -90,7 +90,7 @@ def test_fused_activation_matches_pair_then_swiglu(ops, operand, qname, n):
     up_w = synth.random_packed_weight(qtype, (8, n), k, seed=310 + qtype).cuda()
     x = random_bf16((rows, k), seed=n)
     metadata = _metadata(EXPERTS, offsets)
-    activated, gate = torch.ops.torch_ggml_ops.grouped_mmq_swiglu.default(x, None, gate_w, up_w, *metadata, qtype, n)
+    activated, gate, _kept_up = torch.ops.torch_ggml_ops.grouped_mmq_swiglu.default(x, None, gate_w, up_w, *metadata, qtype, n)
     plain_gate, plain_up = tgo.grouped_mmq_pair(x, gate_w, up_w, *metadata, qtype, n)
     torch.testing.assert_close(gate, plain_gate, rtol=0, atol=0)
     assert_matches_f32_reference(activated, _expected(plain_gate, plain_up), accumulate_noise=1e-6)
@@ -120,14 +120,16 @@ def test_extreme_gates_saturate_cleanly(ops):
     up_w = synth.random_packed_weight(qtype, (1, n), k, seed=52).cuda()
     x = random_bf16((40, k), seed=53, scale=3000.0)
     metadata = _metadata([0], [40])
-    activated, gate = torch.ops.torch_ggml_ops.grouped_mmq_swiglu.default(x, None, gate_w, up_w, *metadata, qtype, n)
+    activated, gate, _kept_up = torch.ops.torch_ggml_ops.grouped_mmq_swiglu.default(x, None, gate_w, up_w, *metadata, qtype, n)
     _, up = tgo.grouped_mmq_pair(x, gate_w, up_w, *metadata, qtype, n)
     assert torch.isfinite(activated).all() and gate.float().abs().max() > 100.0
     assert_matches_f32_reference(activated, _expected(gate, up), accumulate_noise=1e-6)
 
 
 @pytest.mark.parametrize("gathered", (False, True))
-def test_gradient_matches_the_unfused_chain(ops, gathered):
+def test_gradient_matches_the_unfused_chain(ops, operand, gathered):
+    """(with the scaled operands the operator keeps the up projection for the backward pass, otherwise it computes it
+    again there: both routes are compared with the unfused chain)"""
     tgo, synth = ops
     qtype, n, k, experts = 13, 128, 512, 6
     gate_w = synth.random_packed_weight(qtype, (experts, n), k, seed=61).cuda()
@@ -141,7 +143,11 @@ def test_gradient_matches_the_unfused_chain(ops, gathered):
     grad = random_bf16((tokens * top_k, n), seed=65)
 
     fused_in = source.clone().requires_grad_(True)
-    tgo.grouped_mmq_swiglu(fused_in, gate_w, up_w, indices, offsets, qtype, n, row_index if gathered else None).backward(grad)
+    activated, _, kept_up = torch.ops.torch_ggml_ops.grouped_mmq_swiglu.default(
+        fused_in, row_index if gathered else None, gate_w, up_w, indices, offsets, qtype, n
+    )
+    assert kept_up.shape == ((tokens * top_k, n) if operand == "scaled" else (0, n))
+    activated.backward(grad)
 
     plain_in = source.clone().requires_grad_(True)
     if gathered:

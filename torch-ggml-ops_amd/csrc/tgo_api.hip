@@ -487,6 +487,7 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
                       "grouped mmq_forward launch"));
     if (swiglu && !fused) {
         TGO_TRY(check_hip(tgo::launch_swiglu_rows(static_cast<const uint16_t *>(output_first),
+                                                  static_cast<const uint16_t *>(output_second),
                                                   static_cast<uint16_t *>(output_second), rows * out_features, hip_stream),
                           "swiglu launch"));
     }
@@ -534,6 +535,18 @@ int tgo_grouped_mmq_swiglu(const void * input_bf16, const int64_t * row_index, i
     return grouped_forward(input_bf16, row_index, input_rows, packed_gate, packed_up, output_gate, output_activated,
                            expert_indices, expert_offsets, workspace, rows, in_features, out_features, num_experts,
                            num_groups, quant_type, stream, true);
+}
+
+int tgo_swiglu_rows(const void * gate_bf16, const void * up_bf16, void * activated_bf16, int64_t count, void * stream) {
+    if (count <= 0) {
+        return fail(TGO_ERR_INVALID, "count must be positive; got %lld", static_cast<long long>(count));
+    }
+    if (gate_bf16 == nullptr || up_bf16 == nullptr || activated_bf16 == nullptr) {
+        return fail(TGO_ERR_INVALID, "gate, up and activated must not be null");
+    }
+    return check_hip(tgo::launch_swiglu_rows(static_cast<const uint16_t *>(gate_bf16), static_cast<const uint16_t *>(up_bf16),
+                                             static_cast<uint16_t *>(activated_bf16), count, static_cast<hipStream_t>(stream)),
+                     "swiglu launch");
 }
 
 int tgo_swiglu_backward(const void * gate_bf16, const void * up_bf16, const void * grad_activated_bf16,

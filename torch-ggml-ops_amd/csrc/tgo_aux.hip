@@ -538,29 +538,31 @@ __global__ __launch_bounds__(256) void moe_combine_kernel(const uint16_t * __res
     *reinterpret_cast<uint4 *>(out + token * features + feature) = packed;
 }
 
-// activated[i] = bf16(silu(gate[i]) * up[i]) with the up projection stored where the result goes: the second pass of
-// a SwiGLU pair whose multiply kernel has no fused epilogue.  Eight values per thread and step when both tensors
-// start on a 16-byte boundary.
-__global__ __launch_bounds__(256) void swiglu_rows_kernel(const uint16_t * __restrict__ gate, uint16_t * up_then_activated,
-                                                           int64_t count, int vector) {
+// activated[i] = bf16(silu(gate[i]) * up[i]): the second pass of a SwiGLU pair whose multiply kernel has no fused
+// epilogue.  `activated` may be the tensor that holds the up projection (the value is read before it is replaced).
+// Eight values per thread and step when all three tensors start on a 16-byte boundary.
+__global__ __launch_bounds__(256) void swiglu_rows_kernel(const uint16_t * __restrict__ gate, const uint16_t * up,
+                                                           uint16_t * activated, int64_t count, int vector) {
     const int64_t stride = static_cast<int64_t>(gridDim.x) * 256;
     const int64_t first = static_cast<int64_t>(blockIdx.x) * 256 + threadIdx.x;
     const int64_t pieces = vector != 0 ? count / 8 : 0;
     for (int64_t piece = first; piece < pieces; piece += stride) {
-        uint4 * slot = reinterpret_cast<uint4 *>(up_then_activated) + piece;
-        *slot = swiglu_bf16x8(reinterpret_cast<const uint4 *>(gate)[piece], *slot);
+        reinterpret_cast<uint4 *>(activated)[piece] =
+            swiglu_bf16x8(reinterpret_cast<const uint4 *>(gate)[piece], reinterpret_cast<const uint4 *>(up)[piece]);
     }
     for (int64_t index = pieces * 8 + first; index < count; index += stride) {
-        up_then_activated[index] = swiglu_bf16(gate[index], up_then_activated[index]);
+        activated[index] = swiglu_bf16(gate[index], up[index]);
     }
 }
 
-hipError_t launch_swiglu_rows(const uint16_t * gate, uint16_t * up_then_activated, int64_t count, hipStream_t stream) {
-    const int vector = (reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up_then_activated)) % 16 == 0;
+hipError_t launch_swiglu_rows(const uint16_t * gate, const uint16_t * up, uint16_t * activated, int64_t count,
+                              hipStream_t stream) {
+    const int vector =
+        (reinterpret_cast<uintptr_t>(gate) | reinterpret_cast<uintptr_t>(up) | reinterpret_cast<uintptr_t>(activated)) % 16 == 0;
     const int64_t blocks = (count / (vector != 0 ? 8 : 1) + 255) / 256;
     const ProfileScope scope(2, stream);
     swiglu_rows_kernel<<<static_cast<unsigned>(blocks < 1 ? 1 : blocks > 8 * 256 * 8 ? 8 * 256 * 8 : blocks), 256, 0, stream>>>(
-        gate, up_then_activated, count, vector);
+        gate, up, activated, count, vector);
     return hipGetLastError();
 }
 

@@ -234,7 +234,8 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
                                 int64_t in_features, hipStream_t stream, const int64_t * gather = nullptr,
                                 int64_t input_rows = 0, const TaskBuild * build = nullptr);
 // up_then_activated[i] = swiglu(gate[i], up_then_activated[i]) over `count` bf16 values (timed with the forward kernels).
-hipError_t launch_swiglu_rows(const uint16_t * gate, uint16_t * up_then_activated, int64_t count, hipStream_t stream);
+hipError_t launch_swiglu_rows(const uint16_t * gate, const uint16_t * up, uint16_t * activated, int64_t count,
+                              hipStream_t stream);   // (`activated` may be `up`)
 // out[t, :] = sum of rows[order[i], :] over i in [starts[t], starts[t + 1]), in list order (fp32, one rounding).
 hipError_t launch_rows_to_tokens(const uint16_t * rows, const int64_t * order, const int64_t * starts, uint16_t * out,
                                  int tokens, int64_t num_rows, int features, hipStream_t stream);

@@ -47,6 +47,7 @@ lib.tgo_mmq_grad_input.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _int, _p]
 lib.tgo_grouped_mmq_forward.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
 lib.tgo_grouped_mmq_forward_gathered.argtypes = [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
 lib.tgo_grouped_mmq_swiglu.argtypes = [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
+lib.tgo_swiglu_rows.argtypes = [_p, _p, _p, _i64, _p]
 lib.tgo_swiglu_backward.argtypes = [_p, _p, _p, _p, _p, _p, _i64, _p]
 lib.tgo_rows_to_tokens.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _p]
 lib.tgo_moe_combine.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]
@@ -84,6 +85,7 @@ EXPORTS = (
     "tgo_grouped_mmq_forward",
     "tgo_grouped_mmq_forward_gathered",
     "tgo_grouped_mmq_swiglu",
+    "tgo_swiglu_rows",
     "tgo_swiglu_backward",
     "tgo_rows_to_tokens",
     "tgo_moe_combine",

@@ -231,6 +231,32 @@ def measure_decode(args, device) -> dict:
             graph.replay()
         torch.cuda.synchronize()
         graph_elapsed = time.perf_counter() - graph_start
+        # the whole layer from token activations and the router's choices (tgo.moe_layer: routing, gate+up with the
+        # activation, down projection, weighted return to the tokens), replayed from a graph
+        hidden = torch.randn(tokens, 2048, device=device, generator=generator).to(torch.bfloat16)
+        slot_experts = torch.stack([torch.randperm(experts, device=device, generator=generator)[:top_k] for _ in range(tokens)])
+        slot_weights = torch.softmax(torch.randn(tokens, top_k, device=device, generator=generator), dim=1)
+
+        def layer():
+            return tgo.moe_layer(hidden, slot_experts, slot_weights, gate, up, down, synth.IQ2_S, synth.Q6_K, 512)
+
+        with torch.no_grad():
+            capture_stream.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(capture_stream):
+                layer()
+            torch.cuda.current_stream().wait_stream(capture_stream)
+            torch.cuda.synchronize()
+            layer_graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(layer_graph, stream=capture_stream):
+                layer()
+            for _ in range(args.warmup):
+                layer_graph.replay()
+            torch.cuda.synchronize()
+            layer_start = time.perf_counter()
+            for _ in range(args.steps):
+                layer_graph.replay()
+            torch.cuda.synchronize()
+            layer_elapsed = time.perf_counter() - layer_start
         active = sum(r[1].numel() for r in routings) / 8
         weight_bytes = active * (2 * 512 * 8 * 82 + 2048 * 2 * 210)
         report[f"T{tokens}"] = {
@@ -238,6 +264,7 @@ def measure_decode(args, device) -> dict:
             "weight_MB": weight_bytes / 1e6,
             "us_per_layer_call": elapsed / args.steps * 1e6,
             "us_per_layer_call_graph_replay": graph_elapsed / args.steps * 1e6,
+            "us_per_moe_layer_graph_replay": layer_elapsed / args.steps * 1e6,
             "GBps_end_to_end": weight_bytes / (elapsed / args.steps) / 1e9,
             "gemv_kernel_us_per_step": kernel_ms / args.steps * 1e3,
             "quantize_kernel_us_per_step": quantize_ms / args.steps * 1e3,

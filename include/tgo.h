@@ -186,8 +186,8 @@ int tgo_grouped_mmq_forward_gathered(const void * input_bf16, const int64_t * ro
  * operands the up projection is never written and no activation kernel re-reads the pair; with the scaled
  * operands of large calls the up projection passes through output_activated and an elementwise launch
  * replaces it (same values; still faster than the other kinds at that size).  `row_index` may be NULL (rows are input rows) or the
- * gather index of tgo_grouped_mmq_forward_gathered.  Same workspace as tgo_grouped_mmq_forward.  Always runs
- * the MFMA kernel family.  No counterpart in the reference, whose pair operator returns both projections
+ * gather index of tgo_grouped_mmq_forward_gathered.  Same workspace as tgo_grouped_mmq_forward.  Calls of
+ * decode size run the pair in the decode-regime kernels and the same elementwise launch.  No counterpart in the reference, whose pair operator returns both projections
  * (grouped_mmq_pair_cuda, csrc/mmq_hip.cu:1054-1193) and leaves the activation to the caller. */
 int tgo_grouped_mmq_swiglu(const void * input_bf16, const int64_t * row_index, int64_t input_rows,
                            const void * packed_gate, const void * packed_up, void * output_gate,
@@ -211,6 +211,20 @@ int tgo_swiglu_rows(const void * gate_bf16, const void * up_bf16, void * activat
  * (csrc/mmq_hip.cu:1054-1193). */
 int tgo_swiglu_backward(const void * gate_bf16, const void * up_bf16, const void * grad_activated_bf16,
                         const void * grad_gate_bf16, void * d_gate_bf16, void * d_up_bf16, int64_t count, void * stream);
+
+/* Routing of a small batch in one launch: the [tokens, top_k] expert choices sorted by expert (stable), as the
+ * metadata the grouped entry points take, with one group per expert:
+ *   slot_rows int64 [tokens * top_k]       sorted row of each (token, choice) slot; -1 for an expert outside [0, num_experts)
+ *   row_index int64 [tokens * top_k]       token of each sorted row (the gather index of the gathered entry points);
+ *                                          -1 behind the last row
+ *   expert_indices int64 [num_experts]     0, 1, 2, ...
+ *   expert_offsets int32 [num_experts]     rows of experts 0..e
+ * At most TGO_ROUTE_SMALL_LIMIT slots and experts (one workgroup sorts them); larger batches are sorted by the caller.
+ * No counterpart in the reference, whose callers sort with tensor operations (torch_ggml_ops/grouped_mmq.py:216 takes
+ * the sorted metadata); at decode sizes those operations are a dozen launches, more than the layer's own. */
+#define TGO_ROUTE_SMALL_LIMIT 4096
+int tgo_route_small(const int64_t * slot_experts, int64_t tokens, int64_t top_k, int64_t num_experts, int64_t * row_index,
+                    int64_t * slot_rows, int64_t * expert_indices, int32_t * expert_offsets, void * stream);
 
 /* The row gather of the gathered entry points run backwards: the gradients of the sorted rows summed per token,
  *   output[t, :] = bf16( sum of rows[order[i], :] for starts[t] <= i < starts[t + 1] )      (t < tokens)

@@ -44,6 +44,26 @@ def test_route_sorts_slots_by_expert(ops):
     assert indices.tolist() == list(range(9)) and offsets.dtype == torch.int32
 
 
+@pytest.mark.parametrize("tokens,top_k,experts", ((1, 1, 1), (1, 8, 256), (8, 8, 256), (512, 8, 256), (3, 5, 4096),
+                                                    (300, 7, 3), (513, 8, 256), (1000, 8, 64)))
+def test_route_of_any_size_is_the_stable_sort(ops, tokens, top_k, experts):
+    """Up to 4096 slots are sorted by one kernel launch (tgo_route_small), more by tensor operations: either way the
+    result is the stable sort by expert (numpy's), with one group per expert."""
+    tgo, _ = ops
+    generator = np.random.default_rng(tokens * 31 + experts)
+    flat = generator.integers(0, experts, size=tokens * top_k)
+    if tokens * top_k > 20:
+        flat[5:15] = flat[5]          # a run of one expert
+    slot_experts = torch.from_numpy(flat.reshape(tokens, top_k)).cuda()
+    row_index, slot_rows, indices, offsets = tgo.route(slot_experts, experts)
+    order = np.argsort(flat, kind="stable")
+    assert row_index.dtype == torch.int64 and slot_rows.dtype == torch.int64 and slot_rows.shape == (tokens, top_k)
+    assert np.array_equal(row_index.cpu().numpy(), order // top_k)
+    assert np.array_equal(slot_rows.reshape(-1).cpu().numpy()[order], np.arange(flat.size))
+    assert np.array_equal(offsets.cpu().numpy(), np.cumsum(np.bincount(flat, minlength=experts)))
+    assert indices.tolist() == list(range(experts)) and offsets.dtype == torch.int32 and indices.dtype == torch.int64
+
+
 @pytest.mark.parametrize("tokens,top_k,features", ((1, 1, 8), (7, 3, 200), (64, 8, 2048), (5, 6, 4104)))
 def test_combine_matches_float64(ops, tokens, top_k, features):
     tgo, _ = ops

@@ -446,12 +446,20 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
     }
     hipStream_t hip_stream = static_cast<hipStream_t>(stream);
     const int64_t bytes_per_expert = out_features * (in_features / tgo::QK_K) * tgo::block_bytes(quant_type);
-    // (the fused SwiGLU epilogue exists in the MFMA kernel only)
-    const bool gemv = !swiglu && tgo::use_gemv(rows, num_groups);
+    // SwiGLU: the int8 and exact-fp16 matrix-core kernels have the fused epilogue; after the decode-regime kernels and
+    // the scaled-operand kernel, which store both projections (the up projection where the result goes), an
+    // elementwise pass finishes -- for calls of decode size that costs far less than leaving their kernel family
+    const auto finish_swiglu = [&]() {
+        return check_hip(tgo::launch_swiglu_rows(static_cast<const uint16_t *>(output_first),
+                                                 static_cast<const uint16_t *>(output_second),
+                                                 static_cast<uint16_t *>(output_second), rows * out_features, hip_stream),
+                         "swiglu launch");
+    };
+    const bool gemv = tgo::use_gemv(rows, num_groups);
     if (gemv && tgo::gemv_fuses(quant_type, rows, num_groups)) {
         // one launch: the decode-regime kernels of these formats quantize their activations and find their tasks
         // themselves
-        return check_hip(tgo::launch_mmq_gemv_fused(
+        TGO_TRY(check_hip(tgo::launch_mmq_gemv_fused(
                              static_cast<const uint8_t *>(packed_first), static_cast<const uint8_t *>(packed_second),
                              bytes_per_expert, static_cast<const uint16_t *>(input_bf16), row_index,
                              row_index != nullptr ? input_rows : rows, expert_indices, expert_offsets,
@@ -459,12 +467,13 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
                              static_cast<uint16_t *>(output_first), static_cast<uint16_t *>(output_second),
                              static_cast<int>(rows), static_cast<int>(in_features), static_cast<int>(out_features),
                              quant_type, hip_stream),
-                         "grouped mmq_forward launch");
+                         "grouped mmq_forward launch"));
+        return swiglu ? finish_swiglu() : TGO_OK;
     }
     const int operand_kind = tgo::forward_operand_kind(quant_type, rows, out_features, packed_second != nullptr ? 2 : 1);
-    // the scaled-operand kernel has no SwiGLU epilogue: it stores both projections (the up projection where the
-    // result goes) and an elementwise pass finishes, which costs less than the other kinds' kernels lose to it
-    const bool fused = swiglu && operand_kind != tgo::OPERAND_SCALED;
+    // (the scaled-operand kernel without the epilogue plus the elementwise pass costs less than the other kinds'
+    // kernels lose to it)
+    const bool fused = swiglu && !gemv && operand_kind != tgo::OPERAND_SCALED;
     const tgo::Q8Workspace view = tgo::q8_workspace_view(workspace, rows, in_features, gemv, operand_kind);
     void * task_base = static_cast<char *>(workspace) + (tgo::q8_workspace_bytes(rows, in_features) + 15) / 16 * 16;
     const int row_tile = gemv ? tgo::GEMV_ROW_TILE : tgo::forward_row_tile(quant_type, view.operand_kind());
@@ -485,13 +494,7 @@ static int grouped_forward(const void * input_bf16, const int64_t * row_index, i
                              static_cast<uint16_t *>(output_second), &tasks, static_cast<int>(rows),
                              static_cast<int>(in_features), static_cast<int>(out_features), quant_type, hip_stream),
                       "grouped mmq_forward launch"));
-    if (swiglu && !fused) {
-        TGO_TRY(check_hip(tgo::launch_swiglu_rows(static_cast<const uint16_t *>(output_first),
-                                                  static_cast<const uint16_t *>(output_second),
-                                                  static_cast<uint16_t *>(output_second), rows * out_features, hip_stream),
-                          "swiglu launch"));
-    }
-    return TGO_OK;
+    return swiglu && !fused ? finish_swiglu() : TGO_OK;
 }
 
 int tgo_grouped_mmq_forward(const void * input_bf16, const void * packed_first, const void * packed_second,
@@ -590,6 +593,27 @@ int tgo_moe_combine(const void * rows_bf16, const int64_t * slot_rows, const flo
                                              static_cast<int>(top_k), num_rows, static_cast<int>(features),
                                              static_cast<hipStream_t>(stream)),
                      "moe_combine launch");
+}
+
+int tgo_route_small(const int64_t * slot_experts, int64_t tokens, int64_t top_k, int64_t num_experts, int64_t * row_index,
+                    int64_t * slot_rows, int64_t * expert_indices, int32_t * expert_offsets, void * stream) {
+    if (tokens <= 0 || top_k <= 0 || num_experts <= 0) {
+        return fail(TGO_ERR_INVALID, "tokens, top_k and num_experts must be positive");
+    }
+    if (tokens > TGO_ROUTE_SMALL_LIMIT || top_k > TGO_ROUTE_SMALL_LIMIT || tokens * top_k > TGO_ROUTE_SMALL_LIMIT ||
+        num_experts > TGO_ROUTE_SMALL_LIMIT) {
+        return fail(TGO_ERR_INVALID, "tgo_route_small sorts at most %d slots over at most %d experts; got %lld x %lld over %lld",
+                    TGO_ROUTE_SMALL_LIMIT, TGO_ROUTE_SMALL_LIMIT, static_cast<long long>(tokens),
+                    static_cast<long long>(top_k), static_cast<long long>(num_experts));
+    }
+    if (slot_experts == nullptr || row_index == nullptr || slot_rows == nullptr || expert_indices == nullptr ||
+        expert_offsets == nullptr) {
+        return fail(TGO_ERR_INVALID, "slot_experts, row_index, slot_rows, expert_indices and expert_offsets must not be null");
+    }
+    return check_hip(tgo::launch_route_small(slot_experts, static_cast<int>(tokens * top_k), static_cast<int>(top_k),
+                                             static_cast<int>(num_experts), row_index, slot_rows, expert_indices,
+                                             expert_offsets, static_cast<hipStream_t>(stream)),
+                     "route_small launch");
 }
 
 int tgo_rows_to_tokens(const void * rows_bf16, const int64_t * order, const int64_t * starts, void * output_bf16,

@@ -566,6 +566,101 @@ hipError_t launch_swiglu_rows(const uint16_t * gate, const uint16_t * up, uint16
     return hipGetLastError();
 }
 
+// Routing of a small batch in one launch: the (token, choice) slots sorted by expert, stably, by one workgroup.
+//   slot_rows[i]      sorted row of slot i (-1 for a slot whose expert is out of range)
+//   row_index[r]      token of sorted row r (slot / top_k); -1 behind the last row
+//   expert_offsets[e] rows of experts 0..e (the grouped operators' offsets with one group per expert),
+//   expert_indices[e] = e
+// A counting sort: the experts' counts (LDS atomics), their prefix sum, then the slots 256 at a time in slot order,
+// each taking the next place of its expert plus the number of earlier slots of the same expert in its batch of 256.
+// What a decode step otherwise does with a sort and a dozen tensor operations, each a launch of its own.
+constexpr int ROUTE_SMALL_LIMIT = 4096;   // slots and experts one workgroup handles
+__global__ __launch_bounds__(256) void route_small_kernel(const int64_t * __restrict__ slot_experts, int slots, int top_k,
+                                                          int num_experts, int64_t * __restrict__ row_index,
+                                                          int64_t * __restrict__ slot_rows,
+                                                          int64_t * __restrict__ expert_indices,
+                                                          int32_t * __restrict__ expert_offsets) {
+    __shared__ int next_row[ROUTE_SMALL_LIMIT];   // counts, then each expert's next free row
+    __shared__ int batch_expert[256];
+    __shared__ int thread_total[256];
+    const int tid = threadIdx.x;
+    for (int e = tid; e < num_experts; e += 256) {
+        next_row[e] = 0;
+    }
+    for (int i = tid; i < slots; i += 256) {
+        row_index[i] = -1;
+    }
+    __syncthreads();
+    for (int i = tid; i < slots; i += 256) {
+        const int64_t expert = slot_experts[i];
+        if (expert >= 0 && expert < num_experts) {
+            atomicAdd(&next_row[static_cast<int>(expert)], 1);
+        }
+    }
+    __syncthreads();
+    // prefix sum over the experts: a thread owns a run of consecutive experts
+    const int run = (num_experts + 255) / 256;
+    const int first = tid * run;
+    int mine = 0;
+    for (int e = first; e < min(first + run, num_experts); ++e) {
+        mine += next_row[e];
+    }
+    thread_total[tid] = mine;
+    __syncthreads();
+    for (int offset = 1; offset < 256; offset <<= 1) {
+        const int add = tid >= offset ? thread_total[tid - offset] : 0;
+        __syncthreads();
+        thread_total[tid] += add;
+        __syncthreads();
+    }
+    int before = thread_total[tid] - mine;
+    for (int e = first; e < min(first + run, num_experts); ++e) {
+        const int count = next_row[e];
+        next_row[e] = before;
+        before += count;
+        expert_offsets[e] = before;
+        expert_indices[e] = e;
+    }
+    __syncthreads();
+    for (int base = 0; base < slots; base += 256) {
+        const int i = base + tid;
+        int expert = -1;
+        if (i < slots) {
+            const int64_t named = slot_experts[i];
+            expert = named >= 0 && named < num_experts ? static_cast<int>(named) : -1;
+        }
+        batch_expert[tid] = expert;
+        __syncthreads();
+        int row = -1;
+        if (expert >= 0) {
+            int earlier = 0;
+            for (int j = 0; j < tid; ++j) {
+                earlier += batch_expert[j] == expert ? 1 : 0;
+            }
+            row = next_row[expert] + earlier;
+        }
+        __syncthreads();   // (every slot of the batch has read its expert's next row)
+        if (expert >= 0) {
+            atomicAdd(&next_row[expert], 1);
+            row_index[row] = i / top_k;
+        }
+        if (i < slots) {
+            slot_rows[i] = row;
+        }
+        __syncthreads();
+    }
+}
+
+hipError_t launch_route_small(const int64_t * slot_experts, int slots, int top_k, int num_experts, int64_t * row_index,
+                              int64_t * slot_rows, int64_t * expert_indices, int32_t * expert_offsets, hipStream_t stream) {
+    if (slots > ROUTE_SMALL_LIMIT || num_experts > ROUTE_SMALL_LIMIT) {
+        return hipErrorInvalidValue;
+    }
+    route_small_kernel<<<1, 256, 0, stream>>>(slot_experts, slots, top_k, num_experts, row_index, slot_rows, expert_indices,
+                                              expert_offsets);
+    return hipGetLastError();
+}
+
 // The gather of the grouped operators run backwards: out[t, :] = bf16(sum of rows[order[i], :] for i in
 // [starts[t], starts[t + 1])), added in list order in fp32 and rounded once (no atomics: the same bits every time).
 // `order` lists the sorted rows token by token, `starts` where each token's run begins.  Entries that name no row,

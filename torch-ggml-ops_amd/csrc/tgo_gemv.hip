@@ -9,6 +9,7 @@
 // Q4_K / Q5_K tasks of three or more rows use the matrix cores for the dot products instead (gemv_task_k45_mfma).
 // With K of at most four super-blocks several weight rows share a pass (FOLD).  Dense calls of more rows than a
 // task holds are walked in chunks by kernel instantiations of their own.
+#include <algorithm>
 #include <type_traits>
 
 #include "tgo_device.h"
@@ -1597,7 +1598,9 @@ hipError_t launch_mmq_gemv_fused(const uint8_t * packed, const uint8_t * packed_
         args.expert_offsets = expert_offsets;
         args.num_experts = num_experts;
         args.num_groups = num_groups;
-        task_slots = max_tasks_for(rows, num_groups, GEMV_ROWS);
+        // (every task holds at least one row of its own, so a call of few rows over many listed groups -- a router
+        // that lists every expert -- has no more tasks than rows: each slot costs its workgroups a task lookup)
+        task_slots = std::min(max_tasks_for(rows, num_groups, GEMV_ROWS), rows);
     }
     return launch_gemv_by_type(args, task_slots, quant_type, stream);
 }

@@ -236,6 +236,9 @@ hipError_t launch_quantize_q8_1(const uint16_t * input, const Q8Workspace & ws, 
 // up_then_activated[i] = swiglu(gate[i], up_then_activated[i]) over `count` bf16 values (timed with the forward kernels).
 hipError_t launch_swiglu_rows(const uint16_t * gate, const uint16_t * up, uint16_t * activated, int64_t count,
                               hipStream_t stream);   // (`activated` may be `up`)
+// The (token, choice) slots of a small batch sorted by expert in one launch (at most 4096 slots and experts).
+hipError_t launch_route_small(const int64_t * slot_experts, int slots, int top_k, int num_experts, int64_t * row_index,
+                              int64_t * slot_rows, int64_t * expert_indices, int32_t * expert_offsets, hipStream_t stream);
 // out[t, :] = sum of rows[order[i], :] over i in [starts[t], starts[t + 1]), in list order (fp32, one rounding).
 hipError_t launch_rows_to_tokens(const uint16_t * rows, const int64_t * order, const int64_t * starts, uint16_t * out,
                                  int tokens, int64_t num_rows, int features, hipStream_t stream);

@@ -49,6 +49,7 @@ lib.tgo_grouped_mmq_forward_gathered.argtypes = [_p, _p, _i64, _p, _p, _p, _p, _
 lib.tgo_grouped_mmq_swiglu.argtypes = [_p, _p, _i64, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
 lib.tgo_swiglu_rows.argtypes = [_p, _p, _p, _i64, _p]
 lib.tgo_swiglu_backward.argtypes = [_p, _p, _p, _p, _p, _p, _i64, _p]
+lib.tgo_route_small.argtypes = [_p, _i64, _i64, _i64, _p, _p, _p, _p, _p]
 lib.tgo_rows_to_tokens.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _p]
 lib.tgo_moe_combine.argtypes = [_p, _p, _p, _p, _i64, _i64, _i64, _i64, _p]
 lib.tgo_grouped_mmq_grad_input.argtypes = [_p, _p, _p, _p, _p, _p, _p, _p, _i64, _i64, _i64, _i64, _i64, _int, _p]
@@ -87,6 +88,7 @@ EXPORTS = (
     "tgo_grouped_mmq_swiglu",
     "tgo_swiglu_rows",
     "tgo_swiglu_backward",
+    "tgo_route_small",
     "tgo_rows_to_tokens",
     "tgo_moe_combine",
     "tgo_grouped_mmq_grad_input",

@@ -250,6 +250,28 @@ def grouped_mmq_combine(
     return output
 
 
+ROUTE_SMALL_LIMIT = 4096   # TGO_ROUTE_SMALL_LIMIT
+
+
+def _route_small(slot_experts: torch.Tensor, num_experts: int):
+    """``route`` for a decode-sized batch as one kernel (``tgo_route_small``) instead of a sort and a dozen small
+    tensor operations, which at that size cost more than the layer's own launches.  Same results."""
+    tokens, top_k = slot_experts.shape
+    device = slot_experts.device
+    row_index = torch.empty(tokens * top_k, dtype=torch.int64, device=device)
+    slot_rows = torch.empty((tokens, top_k), dtype=torch.int64, device=device)
+    expert_indices = torch.empty(num_experts, dtype=torch.int64, device=device)
+    expert_offsets = torch.empty(num_experts, dtype=torch.int32, device=device)
+    with torch.cuda.device(device):
+        _native.check(
+            _native.lib.tgo_route_small(
+                slot_experts.data_ptr(), tokens, top_k, num_experts, row_index.data_ptr(), slot_rows.data_ptr(),
+                expert_indices.data_ptr(), expert_offsets.data_ptr(), torch.cuda.current_stream(device).cuda_stream,
+            )
+        )
+    return row_index, slot_rows, expert_indices, expert_offsets
+
+
 def route(slot_experts: torch.Tensor, num_experts: int):
     """Sorts the ``[tokens, top_k]`` expert choices by expert (stable, no host synchronisation).
 
@@ -258,6 +280,8 @@ def route(slot_experts: torch.Tensor, num_experts: int):
     group per expert (experts without rows are empty groups, which the operators skip).
     """
     tokens, top_k = slot_experts.shape
+    if slot_experts.is_cuda and 0 < tokens * top_k <= ROUTE_SMALL_LIMIT and 0 < num_experts <= ROUTE_SMALL_LIMIT:
+        return _route_small(slot_experts.contiguous(), num_experts)
     flat = slot_experts.reshape(-1)
     order = torch.argsort(flat, stable=True)
     row_index = torch.div(order, top_k, rounding_mode="floor")

@@ -124,6 +124,40 @@ def test_q8_1_quantizer_matches_oracle_bit_for_bit(ops, oracle, rows, k):
     np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
 
 
+@pytest.mark.parametrize("kind", (0, 1))   # TGO_OPERAND_INT8, TGO_OPERAND_HALF: both keep the quants themselves
+def test_q8_1_quantizer_matches_oracle_for_every_amax(ops, oracle, kind):
+    """Activations are bf16, so a block's amax is one of 2^15 values: every one between 2^-100 and 2^100 (and zero)
+    heads a block here, followed by 31 fractions of it of both signs, and quants, scales (d = amax / 127, with
+    127 / amax behind the quants) and sums must equal the oracle's bit for bit."""
+    _, native, _ = ops
+    exponents = np.arange(127 - 100, 127 + 101, dtype=np.uint32)
+    amax_bits = np.concatenate([[0], ((exponents[:, None] << 7) | np.arange(128, dtype=np.uint32)[None, :]).reshape(-1)])
+    blocks = amax_bits.size
+    rows = (blocks + 63) // 64
+    amax_bits = np.concatenate([amax_bits, np.full(rows * 64 - blocks, 0x3F80, dtype=np.uint32)])
+    amax = torch.from_numpy((amax_bits << 16).astype(np.uint32).view(np.float32).copy()).cuda()
+    generator = torch.Generator(device="cuda").manual_seed(5)
+    factors = torch.rand(rows * 64, 32, device="cuda", generator=generator) * 2.0 - 1.0
+    factors[:, 0] = 1.0
+    factors[:, 1] = -1.0
+    factors[:, 2:10] = torch.tensor([0.5, -0.5, 1.5 / 127, 2.5 / 127, -63.5 / 127, 126.5 / 127, 0.0, -0.0], device="cuda")
+    x = (amax[:, None] * factors).to(torch.bfloat16).reshape(rows, 2048).contiguous()
+    k = 2048
+    workspace = torch.empty(native.lib.tgo_q8_workspace_bytes(rows, k), dtype=torch.uint8, device="cuda")
+    native.check(native.lib.tgo_quantize_q8_1_as(x.data_ptr(), workspace.data_ptr(), rows, k, kind, None))
+    q = torch.empty(rows, k, dtype=torch.int8, device="cuda")
+    d = torch.empty(rows, k // 32, dtype=torch.float32, device="cuda")
+    s = torch.empty(rows, k // 32, dtype=torch.float32, device="cuda")
+    native.check(
+        native.lib.tgo_q8_workspace_unpack(workspace.data_ptr(), q.data_ptr(), d.data_ptr(), s.data_ptr(), rows, k, None)
+    )
+    torch.cuda.synchronize()
+    q_ref, d_ref, s_ref = oracle.quantize_q8_1(bits(x))
+    np.testing.assert_array_equal(d.cpu().numpy().view(np.uint32), d_ref.view(np.uint32))
+    np.testing.assert_array_equal(q.cpu().numpy(), q_ref)
+    np.testing.assert_array_equal(s.cpu().numpy().view(np.uint32), s_ref.view(np.uint32))
+
+
 @pytest.mark.parametrize("qname", tuple(QTYPES))
 @pytest.mark.parametrize("shape,n", [((3, 43), 37), ((1,), 64), ((16,), 130), ((300,), 96)])
 def test_forward_matches_oracle(ops, oracle, qname, shape, n):

@@ -80,7 +80,7 @@ int tgo_q8_workspace_unpack(const void * workspace, void * q_int8, void * d_f32,
 /* output[rows, out_features] = bf16( input[rows, in_features] x W^T ), activations quantized
  * to q8_1, int8 MFMA dot products per block, fp32 scales and accumulation.
  * Decode-sized calls of Q3_K / Q6_K / IQ2_S (dense: at most 8 rows; grouped: at most 64 rows that
- * average at most 4 per listed group) are a single launch whose workgroups quantize their own rows
+ * average at most 4 per listed group, over at most 1024 listed groups) are a single launch whose workgroups quantize their own rows
  * (same q8_1 arithmetic) and, in the grouped entry points, find their task in the group list; such a
  * call leaves `workspace` untouched.
  * Replaces launch_dense_mmq<type>, csrc/mmq_hip.cu:117-147 (called by mmq_cuda, :587-678). */

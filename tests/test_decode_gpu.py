@@ -148,13 +148,15 @@ def test_skewed_small_batch_listed_with_every_expert(ops, oracle, qname):
     assert_matches_f32_reference(compact, expected)
 
 
+@pytest.mark.parametrize("experts", (700, 1500))
 @pytest.mark.parametrize("qname", ("IQ2_S", "Q6_K", "Q3_K"))
-def test_grouped_decode_finds_tasks_among_many_groups(ops, oracle, qname):
+def test_grouped_decode_finds_tasks_among_many_groups(ops, oracle, qname, experts):
     """Small grouped calls of these formats are one launch whose workgroups look their task up in the group list
     themselves, 256 groups per round: 700 listed groups (nearly all empty, some with more than one task, some naming an
-    expert that does not exist) make the lookup run three rounds, with tasks on both sides of every round's boundary."""
+    expert that does not exist) make the lookup run three rounds, with tasks on both sides of every round's boundary.
+    (1500 listed groups are more than that launch accepts: the same call with the task list built by one workgroup.)"""
     tgo, native, synth = ops
-    qtype, n, k, experts = QTYPES[qname], 40, 512, 700
+    qtype, n, k = QTYPES[qname], 40, 512
     rng = np.random.default_rng(77 + qtype)
     sizes = np.zeros(experts, dtype=np.int64)
     for group, size in ((0, 9), (100, 1), (254, 2), (255, 3), (256, 1), (257, 8), (300, 4), (511, 2), (512, 10),

@@ -281,10 +281,14 @@ hipError_t launch_mmq_gemv(const uint8_t * packed, const uint8_t * packed_second
 // workgroup about as much as its dot products once a task has eight rows; it pays while the call is bound by its
 // launches and their latencies: dense calls of one task, grouped calls of at most 64 rows (measured on a 256-expert
 // layer: 1 token x top-8 32 -> 20 us of kernel time, 8 tokens 52 -> 48 us, 256 rows with 200 in one group 68 -> 101 us).
+// Every workgroup of a fused grouped call reads the whole group list to find its task, so a list far longer than any
+// expert count in use (GEMV_FUSED_GROUPS) keeps the task list that one workgroup builds for all.
 constexpr int GEMV_FUSED_GROUPED_ROWS = 64;
+constexpr int GEMV_FUSED_GROUPS = 1024;
 static inline bool gemv_fuses(int quant_type, int64_t rows, int64_t groups) {
     const bool format = quant_type == 11 || quant_type == 14 || quant_type == 22;   // Q3_K, Q6_K, IQ2_S
-    return format && use_gemv(rows, groups) && rows <= (groups <= 0 ? GEMV_ROW_TILE : GEMV_FUSED_GROUPED_ROWS);
+    return format && use_gemv(rows, groups) && groups <= GEMV_FUSED_GROUPS &&
+           rows <= (groups <= 0 ? GEMV_ROW_TILE : GEMV_FUSED_GROUPED_ROWS);
 }
 hipError_t launch_mmq_gemv_fused(const uint8_t * packed, const uint8_t * packed_second, int64_t bytes_per_expert,
                                  const uint16_t * input, const int64_t * gather, int64_t input_rows,

@@ -253,9 +253,17 @@ def grouped_mmq_combine(
 ROUTE_SMALL_LIMIT = 4096   # TGO_ROUTE_SMALL_LIMIT
 
 
-def _route_small(slot_experts: torch.Tensor, num_experts: int):
+torch.library.define(
+    "torch_ggml_ops::route_small",
+    "(Tensor slot_experts, int num_experts) -> (Tensor, Tensor, Tensor, Tensor)",
+)
+
+
+@torch.library.impl("torch_ggml_ops::route_small", "CUDA")
+def _route_small_device(slot_experts, num_experts):
     """``route`` for a decode-sized batch as one kernel (``tgo_route_small``) instead of a sort and a dozen small
     tensor operations, which at that size cost more than the layer's own launches.  Same results."""
+    slot_experts = slot_experts.to(torch.int64).contiguous()
     tokens, top_k = slot_experts.shape
     device = slot_experts.device
     row_index = torch.empty(tokens * top_k, dtype=torch.int64, device=device)
@@ -272,6 +280,17 @@ def _route_small(slot_experts: torch.Tensor, num_experts: int):
     return row_index, slot_rows, expert_indices, expert_offsets
 
 
+@torch.library.register_fake("torch_ggml_ops::route_small")
+def _route_small_fake(slot_experts, num_experts):
+    tokens, top_k = slot_experts.shape
+    return (
+        slot_experts.new_empty((tokens * top_k,), dtype=torch.int64),
+        slot_experts.new_empty((tokens, top_k), dtype=torch.int64),
+        slot_experts.new_empty((num_experts,), dtype=torch.int64),
+        slot_experts.new_empty((num_experts,), dtype=torch.int32),
+    )
+
+
 def route(slot_experts: torch.Tensor, num_experts: int):
     """Sorts the ``[tokens, top_k]`` expert choices by expert (stable, no host synchronisation).
 
@@ -281,7 +300,7 @@ def route(slot_experts: torch.Tensor, num_experts: int):
     """
     tokens, top_k = slot_experts.shape
     if slot_experts.is_cuda and 0 < tokens * top_k <= ROUTE_SMALL_LIMIT and 0 < num_experts <= ROUTE_SMALL_LIMIT:
-        return _route_small(slot_experts.contiguous(), num_experts)
+        return torch.ops.torch_ggml_ops.route_small.default(slot_experts, int(num_experts))
     flat = slot_experts.reshape(-1)
     order = torch.argsort(flat, stable=True)
     row_index = torch.div(order, top_k, rounding_mode="floor")

@@ -127,3 +127,19 @@ def test_scaled_pair_with_short_groups_replays_bit_identically(ops):
         for got, want in zip(captured, eager):
             assert torch.equal(got, want), f"replay {replay} differs from the eager result"
         assert torch.isfinite(scratch)
+
+
+def test_launch_stream_is_torch_current_stream(ops):
+    """The handle the operators launch on is that of torch's current stream, on the default stream and inside
+    ``torch.cuda.stream(...)``; the device context is only entered when another device is current."""
+    from torch_ggml_ops import _native
+
+    device = torch.device("cuda", torch.cuda.current_device())
+    assert _native.stream_of(device) == torch.cuda.current_stream(device).cuda_stream
+    side = torch.cuda.Stream()
+    with torch.cuda.stream(side):
+        assert _native.stream_of(device) == side.cuda_stream
+    assert _native.stream_of(device) == torch.cuda.current_stream(device).cuda_stream
+    with _native.on_device(device):
+        assert torch.cuda.current_device() == device.index
+    assert _native.stream_of(torch.device("cuda")) == torch.cuda.current_stream().cuda_stream   # no index: torch's own call

@@ -6,8 +6,11 @@ fallback: if it is missing, importing the package fails.
 
 from __future__ import annotations
 
+import contextlib
 import ctypes
 from pathlib import Path
+
+import torch
 
 _LIB_PATH = Path(__file__).resolve().parent / "libtgo_hip.so"
 
@@ -125,6 +128,27 @@ def profile_read(kernel: str) -> tuple[float, int]:
     total, count = ctypes.c_double(0.0), ctypes.c_int64(0)
     check(lib.tgo_profile_read(KERNEL_IDS[kernel], ctypes.byref(total), ctypes.byref(count)))
     return total.value, count.value
+
+
+_raw_stream = getattr(torch._C, "_cuda_getCurrentRawStream", None)
+_current_device = getattr(torch._C, "_cuda_getDevice", None)
+_STAY = contextlib.nullcontext()
+
+
+def stream_of(device: torch.device) -> int:
+    """Handle of torch's current stream on ``device``, the value of ``torch.cuda.current_stream(device).cuda_stream``:
+    taken through torch's raw call where it has one, because building the Stream object costs a decode-sized call a
+    quarter of its host time."""
+    if _raw_stream is not None and device.index is not None:
+        return _raw_stream(device.index)
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+def on_device(device: torch.device):
+    """Context in which ``device`` is the current device; nothing is entered when it already is."""
+    if _current_device is not None and device.index is not None and _current_device() == device.index:
+        return _STAY
+    return torch.cuda.device(device)
 
 
 def check(status: int) -> None:

@@ -92,11 +92,11 @@ def _scatter_to_tokens(grad_rows: torch.Tensor, row_index: torch.Tensor, tokens:
     grad_rows = grad_rows.contiguous()
     order, starts = _token_runs(row_index, tokens)
     out = torch.empty((tokens, grad_rows.shape[1]), dtype=grad_rows.dtype, device=grad_rows.device)
-    with torch.cuda.device(grad_rows.device):
+    with _native.on_device(grad_rows.device):
         _native.check(
             _native.lib.tgo_rows_to_tokens(
                 grad_rows.data_ptr(), order.data_ptr(), starts.data_ptr(), out.data_ptr(), tokens, grad_rows.shape[0],
-                grad_rows.shape[1], torch.cuda.current_stream(grad_rows.device).cuda_stream,
+                grad_rows.shape[1], _native.stream_of(grad_rows.device),
             )
         )
     return out

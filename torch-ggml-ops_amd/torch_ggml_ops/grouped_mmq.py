@@ -36,7 +36,7 @@ torch.library.define(
 
 
 def _stream(tensor: torch.Tensor) -> int:
-    return torch.cuda.current_stream(tensor.device).cuda_stream
+    return _native.stream_of(tensor.device)
 
 
 def _forward(
@@ -56,7 +56,7 @@ def _forward(
         )
         if second[3] != experts or second[5] != bytes_per_expert:
             raise RuntimeError("paired grouped MMQ weights must have identical physical geometry")
-    with torch.cuda.device(input.device):
+    with _native.on_device(input.device):
         first_output = input.new_empty((rows, out_features))
         second_output = input.new_empty((rows, out_features)) if second_weight is not None else None
         workspace_bytes = (
@@ -98,7 +98,7 @@ def _grad_input(
         )
         if (second[0], second[2], second[3], second[4], second[5]) != (rows, out_features, experts, groups, bytes_per_expert):
             raise RuntimeError("paired grouped MMQ backward tensors must have identical physical geometry")
-    with torch.cuda.device(first_grad.device):
+    with _native.on_device(first_grad.device):
         grad_input = (first_grad.new_zeros if zero_fill else first_grad.new_empty)((rows, in_features))
         sources = 2 if second_weight is not None else 1
         workspace = first_grad.new_empty(

@@ -23,13 +23,13 @@ torch.library.define(
 
 
 def _stream(tensor: torch.Tensor) -> int:
-    return torch.cuda.current_stream(tensor.device).cuda_stream
+    return _native.stream_of(tensor.device)
 
 
 @torch.library.impl("torch_ggml_ops::mmq", "CUDA")
 def _mmq_device(input: torch.Tensor, packed_weight: torch.Tensor, quant_type: int, out_features: int) -> torch.Tensor:
     rows, in_features, out_features = _validate.dense(input, packed_weight, quant_type, out_features, backward=False)
-    with torch.cuda.device(input.device):
+    with _native.on_device(input.device):
         output = input.new_empty((*input.shape[:-1], out_features))
         workspace = input.new_empty(
             (_native.lib.tgo_q8_workspace_bytes(rows, in_features),), dtype=torch.uint8
@@ -48,7 +48,7 @@ def _mmq_grad_input_device(
     grad_output: torch.Tensor, packed_weight: torch.Tensor, quant_type: int, in_features: int
 ) -> torch.Tensor:
     rows, in_features, out_features = _validate.dense(grad_output, packed_weight, quant_type, in_features, backward=True)
-    with torch.cuda.device(grad_output.device):
+    with _native.on_device(grad_output.device):
         grad_input = grad_output.new_empty((*grad_output.shape[:-1], in_features))
         workspace = grad_output.new_empty(
             (_native.lib.tgo_dense_grad_workspace_bytes(rows, out_features, in_features, quant_type),), dtype=torch.uint8

@@ -56,12 +56,12 @@ def _check_combine(rows: torch.Tensor, slot_rows: torch.Tensor, slot_weights: to
 def _combine_device(rows, slot_rows, slot_weights):
     _check_combine(rows, slot_rows, slot_weights)
     tokens, top_k = slot_rows.shape
-    with torch.cuda.device(rows.device):
+    with _native.on_device(rows.device):
         output = rows.new_empty((tokens, rows.shape[1]))
         _native.check(
             _native.lib.tgo_moe_combine(
                 rows.data_ptr(), slot_rows.data_ptr(), slot_weights.data_ptr(), output.data_ptr(),
-                tokens, top_k, rows.shape[0], rows.shape[1], torch.cuda.current_stream(rows.device).cuda_stream,
+                tokens, top_k, rows.shape[0], rows.shape[1], _native.stream_of(rows.device),
             )
         )
     return output
@@ -133,7 +133,7 @@ def _grad_input_weighted_device(
         _fail("row_weight must be a contiguous torch.float32 tensor with one entry per row")
     if row_weight.device != grad_tokens.device:
         _fail("all grouped MMQ backward tensors must be on the same device")
-    with torch.cuda.device(grad_tokens.device):
+    with _native.on_device(grad_tokens.device):
         # (rows that no valid group covers stay unwritten, as for grouped_mmq_grad_input)
         grad_input = grad_tokens.new_empty((rows, in_features))
         workspace = grad_tokens.new_empty(
@@ -144,7 +144,7 @@ def _grad_input_weighted_device(
                 grad_tokens.data_ptr(), row_token.data_ptr(), row_weight.data_ptr(), tokens,
                 packed_weight.data_ptr(), grad_input.data_ptr(), expert_indices.data_ptr(), expert_offsets.data_ptr(),
                 workspace.data_ptr(), rows, out_features, in_features, experts, groups, int(quant_type),
-                torch.cuda.current_stream(grad_tokens.device).cuda_stream,
+                _native.stream_of(grad_tokens.device),
             )
         )
     return grad_input
@@ -270,11 +270,11 @@ def _route_small_device(slot_experts, num_experts):
     slot_rows = torch.empty((tokens, top_k), dtype=torch.int64, device=device)
     expert_indices = torch.empty(num_experts, dtype=torch.int64, device=device)
     expert_offsets = torch.empty(num_experts, dtype=torch.int32, device=device)
-    with torch.cuda.device(device):
+    with _native.on_device(device):
         _native.check(
             _native.lib.tgo_route_small(
                 slot_experts.data_ptr(), tokens, top_k, num_experts, row_index.data_ptr(), slot_rows.data_ptr(),
-                expert_indices.data_ptr(), expert_offsets.data_ptr(), torch.cuda.current_stream(device).cuda_stream,
+                expert_indices.data_ptr(), expert_offsets.data_ptr(), _native.stream_of(device),
             )
         )
     return row_index, slot_rows, expert_indices, expert_offsets

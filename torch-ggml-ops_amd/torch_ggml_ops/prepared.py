@@ -37,7 +37,7 @@ torch.library.define(
 
 
 def _stream(tensor: torch.Tensor) -> int:
-    return torch.cuda.current_stream(tensor.device).cuda_stream
+    return _native.stream_of(tensor.device)
 
 
 def _workspace_kind(operand: str) -> int:
@@ -59,7 +59,7 @@ def _activation_shape(input: torch.Tensor) -> tuple[int, int]:
 def _quantize_device(input: torch.Tensor, operand: str = "") -> torch.Tensor:
     rows, in_features = _activation_shape(input)
     kind = _workspace_kind(operand)
-    with torch.cuda.device(input.device):
+    with _native.on_device(input.device):
         workspace = input.new_empty((_native.lib.tgo_q8_workspace_bytes(rows, in_features),), dtype=torch.uint8)
         _native.check(
             _native.lib.tgo_quantize_q8_1_as(
@@ -91,7 +91,7 @@ def _mmq_prepared_device(
         raise RuntimeError(
             f"workspace holds {workspace.numel()} bytes; quantize_q8_1 of [{rows}, {in_features}] writes {expected}"
         )
-    with torch.cuda.device(workspace.device):
+    with _native.on_device(workspace.device):
         output = workspace.new_empty((rows, out_features), dtype=torch.bfloat16)
         _native.check(
             _native.lib.tgo_mmq_forward_prepared_as(

@@ -49,11 +49,11 @@ def _swiglu_device(
             input, gate_packed_weight, up_packed_weight, expert_indices, expert_offsets, quant_type, out_features, row_index
         )
         activated = torch.empty_like(up)
-        with torch.cuda.device(gate.device):
+        with _native.on_device(gate.device):
             _native.check(
                 _native.lib.tgo_swiglu_rows(
                     gate.data_ptr(), up.data_ptr(), activated.data_ptr(), gate.numel(),
-                    torch.cuda.current_stream(gate.device).cuda_stream,
+                    _native.stream_of(gate.device),
                 )
             )
         return activated, gate, up
@@ -81,11 +81,11 @@ def _activation_backward(gate, up, grad_activated, grad_gate):
     tensors = [gate, up, grad_activated] + ([] if grad_gate is None else [grad_gate])
     gate, up, grad_activated, *rest = [t.contiguous() for t in tensors]
     d_gate, d_up = torch.empty_like(gate), torch.empty_like(gate)
-    with torch.cuda.device(gate.device):
+    with _native.on_device(gate.device):
         _native.check(
             _native.lib.tgo_swiglu_backward(
                 gate.data_ptr(), up.data_ptr(), grad_activated.data_ptr(), rest[0].data_ptr() if rest else None,
-                d_gate.data_ptr(), d_up.data_ptr(), gate.numel(), torch.cuda.current_stream(gate.device).cuda_stream,
+                d_gate.data_ptr(), d_up.data_ptr(), gate.numel(), _native.stream_of(gate.device),
             )
         )
     return d_gate, d_up

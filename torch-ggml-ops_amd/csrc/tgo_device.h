@@ -246,6 +246,34 @@ TGO_DEVICE void expand_iq2s_grid(uint2 * grid_lds, int tid, int nthreads) {
     }
 }
 
+// The same in two steps for kernels that have other memory round trips to start first: the packed entries are
+// requested early (ENTRIES_PER_THREAD = 1024 / threads of the block) and expanded once the other requests are out.
+template <int ENTRIES_PER_THREAD>
+TGO_DEVICE void request_iq2s_grid(uint32_t (&packed)[ENTRIES_PER_THREAD], int tid) {
+#pragma unroll
+    for (int j = 0; j < ENTRIES_PER_THREAD; ++j) {
+        packed[j] = tgo_iq2s_packed[tid + j * (TGO_IQ2S_GRID_ENTRIES / ENTRIES_PER_THREAD)];
+    }
+}
+template <int ENTRIES_PER_THREAD>
+TGO_DEVICE void expand_iq2s_grid(uint2 * grid_lds, const uint32_t (&packed)[ENTRIES_PER_THREAD], int tid) {
+#pragma unroll
+    for (int j = 0; j < ENTRIES_PER_THREAD; ++j) {
+        uint32_t words[2];
+#pragma unroll
+        for (int w = 0; w < 2; ++w) {
+            uint32_t word = 0;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const uint32_t digit = (packed[j] >> (2 * (4 * w + e))) & 3u;
+                word |= (8u + 17u * digit + (digit >> 1)) << (8 * e);
+            }
+            words[w] = word;
+        }
+        grid_lds[tid + j * (TGO_IQ2S_GRID_ENTRIES / ENTRIES_PER_THREAD)] = make_uint2(words[0], words[1]);
+    }
+}
+
 // Copies `nrows` super-blocks (block column `kb` of consecutive weight rows starting at `row0`) into
 // LDS slots of RAW_PITCH bytes.  Rows past `row_limit - 1` re-read the last valid row; callers mask
 // what they compute from them.

@@ -1403,6 +1403,12 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a
     const bool second = n_group >= a.n_groups;
     n_group -= second ? a.n_groups : 0;
 
+    // the codebook's packed entries travel while the task is looked up
+    constexpr int GRID_PER_THREAD = TGO_IQ2S_GRID_ENTRIES / GEMV_THREADS;
+    uint32_t packed_grid[TYPE == IQ2_S ? GRID_PER_THREAD : 1];
+    if constexpr (TYPE == IQ2_S) {
+        request_iq2s_grid<GRID_PER_THREAD>(packed_grid, tid);
+    }
     int expert = 0, row_start = 0, row_end = a.rows;
     if constexpr (FUSED) {
         if (a.expert_offsets != nullptr && !gemv_find_task(a, task, tid, found_task, expert, row_start, row_end)) {
@@ -1423,7 +1429,7 @@ __global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a
     const int n0 = n_group * GEMV_GN;
 
     if constexpr (TYPE == IQ2_S) {
-        expand_iq2s_grid(grid, tid, GEMV_THREADS);
+        expand_iq2s_grid<GRID_PER_THREAD>(grid, packed_grid, tid);
     }
     // a task has 1..GEMV_ROWS rows; a walked dense call has more (every routine starts with a barrier before it
     // touches LDS again)

@@ -260,7 +260,11 @@ def measure_decode(args, device) -> dict:
             torch.cuda.synchronize()
             layer_elapsed = time.perf_counter() - layer_start
         active = sum(r[1].numel() for r in routings) / 8
-        weight_bytes = active * (2 * 512 * 8 * 82 + 2048 * 2 * 210)
+        expert_bytes = 2 * 512 * 8 * 82 + 2048 * 2 * 210
+        weight_bytes = active * expert_bytes
+        # (the whole-layer replay routes every token to top_k different experts drawn uniformly: more experts, and
+        # so more weight bytes, than the skewed routings of the layer calls above)
+        layer_active = int(slot_experts.unique().numel())
         report[f"T{tokens}"] = {
             "active_experts": active,
             "weight_MB": weight_bytes / 1e6,
@@ -268,6 +272,9 @@ def measure_decode(args, device) -> dict:
             "us_per_layer_call_graph_replay": graph_elapsed / replays * 1e6,
             "us_per_moe_layer_graph_replay": layer_elapsed / replays * 1e6,
             "graph_replays_timed": replays,
+            "moe_layer_active_experts": layer_active,
+            "moe_layer_weight_MB": layer_active * expert_bytes / 1e6,
+            "moe_layer_GBps_graph_replay": layer_active * expert_bytes / (layer_elapsed / replays) / 1e9,
             "GBps_end_to_end": weight_bytes / (elapsed / args.steps) / 1e9,
             "gemv_kernel_us_per_step": kernel_ms / args.steps * 1e3,
             "quantize_kernel_us_per_step": quantize_ms / args.steps * 1e3,

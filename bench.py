@@ -213,68 +213,74 @@ def measure_decode(args, device) -> dict:
         _native.lib.tgo_profile_enable(0)
         if launches == 0:
             continue  # too many rows per expert for the GEMV family: that shape belongs to the MFMA benchmark
-        # the same layer call replayed from a HIP graph (one routing): what a serving loop would do about launch cost
-        capture_stream = torch.cuda.Stream()
-        capture_stream.wait_stream(torch.cuda.current_stream())
-        with torch.cuda.stream(capture_stream):
-            step(0)
-        torch.cuda.current_stream().wait_stream(capture_stream)
-        torch.cuda.synchronize()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=capture_stream):
-            step(0)
-        # (a replay is tens of microseconds: enough of them that the closing synchronisation does not set the figure)
-        replays = max(args.steps, 200)
-        for _ in range(args.warmup):
-            graph.replay()
-        torch.cuda.synchronize()
-        graph_start = time.perf_counter()
-        for _ in range(replays):
-            graph.replay()
-        torch.cuda.synchronize()
-        graph_elapsed = time.perf_counter() - graph_start
-        # the whole layer from token activations and the router's choices (tgo.moe_layer: routing, gate+up with the
-        # activation, down projection, weighted return to the tokens), replayed from a graph
-        hidden = torch.randn(tokens, 2048, device=device, generator=generator).to(torch.bfloat16)
-        slot_experts = torch.stack([torch.randperm(experts, device=device, generator=generator)[:top_k] for _ in range(tokens)])
-        slot_weights = torch.softmax(torch.randn(tokens, top_k, device=device, generator=generator), dim=1)
-
-        def layer():
-            return tgo.moe_layer(hidden, slot_experts, slot_weights, gate, up, down, synth.IQ2_S, synth.Q6_K, 512)
-
-        with torch.no_grad():
+        graph_fields = {}
+        if not args.no_graph_replays:
+            # the same layer call replayed from a HIP graph (one routing): what a serving loop would do about launch cost
+            capture_stream = torch.cuda.Stream()
             capture_stream.wait_stream(torch.cuda.current_stream())
             with torch.cuda.stream(capture_stream):
-                layer()
+                step(0)
             torch.cuda.current_stream().wait_stream(capture_stream)
             torch.cuda.synchronize()
-            layer_graph = torch.cuda.CUDAGraph()
-            with torch.cuda.graph(layer_graph, stream=capture_stream):
-                layer()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph, stream=capture_stream):
+                step(0)
+            # (a replay is tens of microseconds: enough of them that the closing synchronisation does not set the figure)
+            replays = max(args.steps, 200)
             for _ in range(args.warmup):
-                layer_graph.replay()
+                graph.replay()
             torch.cuda.synchronize()
-            layer_start = time.perf_counter()
+            graph_start = time.perf_counter()
             for _ in range(replays):
-                layer_graph.replay()
+                graph.replay()
             torch.cuda.synchronize()
-            layer_elapsed = time.perf_counter() - layer_start
+            graph_elapsed = time.perf_counter() - graph_start
+            # the whole layer from token activations and the router's choices (tgo.moe_layer: routing, gate+up with the
+            # activation, down projection, weighted return to the tokens), replayed from a graph
+            hidden = torch.randn(tokens, 2048, device=device, generator=generator).to(torch.bfloat16)
+            slot_experts = torch.stack([torch.randperm(experts, device=device, generator=generator)[:top_k] for _ in range(tokens)])
+            slot_weights = torch.softmax(torch.randn(tokens, top_k, device=device, generator=generator), dim=1)
+
+            def layer():
+                return tgo.moe_layer(hidden, slot_experts, slot_weights, gate, up, down, synth.IQ2_S, synth.Q6_K, 512)
+
+            with torch.no_grad():
+                capture_stream.wait_stream(torch.cuda.current_stream())
+                with torch.cuda.stream(capture_stream):
+                    layer()
+                torch.cuda.current_stream().wait_stream(capture_stream)
+                torch.cuda.synchronize()
+                layer_graph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(layer_graph, stream=capture_stream):
+                    layer()
+                for _ in range(args.warmup):
+                    layer_graph.replay()
+                torch.cuda.synchronize()
+                layer_start = time.perf_counter()
+                for _ in range(replays):
+                    layer_graph.replay()
+                torch.cuda.synchronize()
+                layer_elapsed = time.perf_counter() - layer_start
         active = sum(r[1].numel() for r in routings) / 8
         expert_bytes = 2 * 512 * 8 * 82 + 2048 * 2 * 210
         weight_bytes = active * expert_bytes
-        # (the whole-layer replay routes every token to top_k different experts drawn uniformly: more experts, and
-        # so more weight bytes, than the skewed routings of the layer calls above)
-        layer_active = int(slot_experts.unique().numel())
+        if not args.no_graph_replays:
+            # (the whole-layer replay routes every token to top_k different experts drawn uniformly: more experts, and
+            # so more weight bytes, than the skewed routings of the layer calls above)
+            layer_active = int(slot_experts.unique().numel())
+            graph_fields = {
+                "us_per_layer_call_graph_replay": graph_elapsed / replays * 1e6,
+                "us_per_moe_layer_graph_replay": layer_elapsed / replays * 1e6,
+                "graph_replays_timed": replays,
+                "moe_layer_active_experts": layer_active,
+                "moe_layer_weight_MB": layer_active * expert_bytes / 1e6,
+                "moe_layer_GBps_graph_replay": layer_active * expert_bytes / (layer_elapsed / replays) / 1e9,
+            }
         report[f"T{tokens}"] = {
             "active_experts": active,
             "weight_MB": weight_bytes / 1e6,
             "us_per_layer_call": elapsed / args.steps * 1e6,
-            "us_per_layer_call_graph_replay": graph_elapsed / replays * 1e6,
-            "us_per_moe_layer_graph_replay": layer_elapsed / replays * 1e6,
-            "graph_replays_timed": replays,
-            "moe_layer_active_experts": layer_active,
-            "moe_layer_weight_MB": layer_active * expert_bytes / 1e6,
-            "moe_layer_GBps_graph_replay": layer_active * expert_bytes / (layer_elapsed / replays) / 1e9,
+            **graph_fields,
             "GBps_end_to_end": weight_bytes / (elapsed / args.steps) / 1e9,
             "gemv_kernel_us_per_step": kernel_ms / args.steps * 1e3,
             "quantize_kernel_us_per_step": quantize_ms / args.steps * 1e3,
@@ -723,6 +729,9 @@ def main() -> None:
                         help="decode workload: which cases to run (T1, T4, T8: MoE layer calls; dense: Q3_K [4096,2048] "
                         "single row; big: Q4_K [28672,8192] with 1..16 rows; skewed: 256 rows, 200 of them in one of 57 "
                         "groups, all 256 experts listed)")
+    parser.add_argument("--no-graph-replays", action="store_true",
+                        help="decode workload: leave out the graph replays (profiler runs: per-dispatch averages then "
+                             "cover the eager layer calls only)")
     parser.add_argument("--no-sub-records", action="store_true",
                         help="pair workload only: skip the down-projection and decode sub-records")
     parser.add_argument("--workload", choices=("pair", "decode", "multi", "gathered", "layer", "dense", "down"), default="pair")

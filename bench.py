@@ -227,7 +227,7 @@ def measure_decode(args, device) -> dict:
                 step(0)
             # (a replay is tens of microseconds: enough of them that the closing synchronisation does not set the figure)
             replays = max(args.steps, 200)
-            for _ in range(args.warmup):
+            for _ in range(max(args.warmup, 50)):
                 graph.replay()
             torch.cuda.synchronize()
             graph_start = time.perf_counter()
@@ -253,7 +253,7 @@ def measure_decode(args, device) -> dict:
                 layer_graph = torch.cuda.CUDAGraph()
                 with torch.cuda.graph(layer_graph, stream=capture_stream):
                     layer()
-                for _ in range(args.warmup):
+                for _ in range(max(args.warmup, 50)):
                     layer_graph.replay()
                 torch.cuda.synchronize()
                 layer_start = time.perf_counter()

@@ -199,12 +199,15 @@ def measure_decode(args, device) -> dict:
             tgo.grouped_mmq_pair(x, gate, up, indices, offsets, synth.IQ2_S, 512)
             tgo.grouped_mmq(mid[i % 8], down, indices, offsets, synth.Q6_K, 2048)
 
-        for i in range(args.warmup):
+        # (a layer call is tens of microseconds: timed over enough calls that the first ones, which still grow
+        # torch's allocator pools, and the closing synchronisation do not set the figures)
+        steps, warmup = max(args.steps, 100), max(args.warmup, 20)
+        for i in range(warmup):
             step(i)
         torch.cuda.synchronize()
         _native.lib.tgo_profile_enable(1)
         start = time.perf_counter()
-        for i in range(args.steps):
+        for i in range(steps):
             step(i)
         torch.cuda.synchronize()
         elapsed = time.perf_counter() - start
@@ -279,13 +282,14 @@ def measure_decode(args, device) -> dict:
         report[f"T{tokens}"] = {
             "active_experts": active,
             "weight_MB": weight_bytes / 1e6,
-            "us_per_layer_call": elapsed / args.steps * 1e6,
+            "layer_calls_timed": steps,
+            "us_per_layer_call": elapsed / steps * 1e6,
             **graph_fields,
-            "GBps_end_to_end": weight_bytes / (elapsed / args.steps) / 1e9,
-            "gemv_kernel_us_per_step": kernel_ms / args.steps * 1e3,
-            "quantize_kernel_us_per_step": quantize_ms / args.steps * 1e3,
-            "launches_per_layer_call": launches / args.steps + (2 if quantize_ms > 0 else 0),
-            "GBps_gemv_kernels": weight_bytes / (kernel_ms / args.steps * 1e-3) / 1e9,
+            "GBps_end_to_end": weight_bytes / (elapsed / steps) / 1e9,
+            "gemv_kernel_us_per_step": kernel_ms / steps * 1e3,
+            "quantize_kernel_us_per_step": quantize_ms / steps * 1e3,
+            "launches_per_layer_call": launches / steps + (2 if quantize_ms > 0 else 0),
+            "GBps_gemv_kernels": weight_bytes / (kernel_ms / steps * 1e-3) / 1e9,
         }
     x = torch.randn(1, 2048, device=device, generator=generator).to(torch.bfloat16)
     if "dense" not in cases:

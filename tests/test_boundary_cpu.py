@@ -138,6 +138,37 @@ def test_grouped_validation_messages(package):
         validate.REQUIRE_DEVICE = True
 
 
+def test_second_weight_of_a_pair_is_checked_like_the_first(package):
+    """A second weight with the first one's geometry needs no second pass through the checks; any other goes through
+    them and fails with their message (or with the pair's own, when it is a valid weight of another expert count)."""
+    from torch_ggml_ops.grouped_mmq import _forward
+
+    _, _, validate, synth = package
+    validate.REQUIRE_DEVICE = False
+    try:
+        packed = synth.random_packed_weight(12, (8, 37), 2048, seed=2)
+        other = synth.random_packed_weight(12, (8, 37), 2048, seed=3)
+        assert validate.same_weight_geometry(packed, other)
+        assert not validate.same_weight_geometry(packed, other[:, :, :-1])                  # not contiguous
+        assert not validate.same_weight_geometry(packed, other[:4].contiguous())           # fewer experts
+        assert not validate.same_weight_geometry(packed, other.to(torch.int8))             # another dtype
+        assert not validate.same_weight_geometry(packed, other.reshape(-1)[16:].reshape(-1))   # another shape, offset
+        x = torch.randn(262, 2048).to(torch.bfloat16)
+        experts = torch.tensor([0, 2, 5, 7], dtype=torch.int64)
+        offsets = torch.tensor([1, 128, 257, 262], dtype=torch.int32)
+        cases = [
+            (other[:, :, :-1], "contiguous"),
+            (other[:, :36].contiguous(), "does not match out_features"),
+            (other.to(torch.int8), "torch.uint8"),
+            (other[:4].contiguous(), "identical physical geometry"),
+        ]
+        for second, fragment in cases:
+            with pytest.raises(RuntimeError, match=fragment):
+                _forward(x, packed, second, experts, offsets, 12, 37)
+    finally:
+        validate.REQUIRE_DEVICE = True
+
+
 def test_operator_schemas_and_fake_kernels(package):
     tgo, _, _, _ = package
     ops = torch.ops.torch_ggml_ops

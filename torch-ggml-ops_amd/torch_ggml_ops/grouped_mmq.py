@@ -50,7 +50,7 @@ def _forward(
     input_rows = rows
     if row_index is not None:
         rows = _validate.row_index(row_index, input)
-    if second_weight is not None:
+    if second_weight is not None and not _validate.same_weight_geometry(first_weight, second_weight):
         second = _validate.grouped(
             input, second_weight, expert_indices, expert_offsets, quant_type, out_features, backward=False
         )

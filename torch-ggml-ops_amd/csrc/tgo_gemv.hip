@@ -1382,8 +1382,13 @@ TGO_DEVICE bool gemv_find_task(const GemvArgs & a, int task, int tid, int * shar
 // (every grouped call, every dense call of up to GEMV_ROWS rows) a wave per SIMD if they share the code.
 // FUSED: bf16 activations, quantized by the workgroups themselves (gemv_task), and, for grouped calls, the task looked
 // up in the group list instead of a task list (gemv_find_task): the whole call is this one launch.
+// Three workgroups per CU are asked of the compiler for the fused IQ2_S instances of more than two rows (their eight-row
+// routine alone would take 223 registers and leave room for two): it spills a little in that routine, which few tasks
+// of a decode batch take, and the tasks of one to four rows gain the third workgroup.  The other formats' instances
+// spill three times as much under the same bound and measured slower with it.
 template <int TYPE, int MAX_ROWS, int FOLD, bool WALK = false, bool FUSED = false>
-__global__ __launch_bounds__(GEMV_THREADS) void mmq_gemv_kernel(const GemvArgs a) {
+__global__ __launch_bounds__(GEMV_THREADS, (FUSED && MAX_ROWS > 2 && TYPE == IQ2_S && FOLD == 1) ? 3 : 1)
+void mmq_gemv_kernel(const GemvArgs a) {
     static_assert(!WALK || MAX_ROWS == GEMV_ROWS, "a walked call has full chunks");
     using F = Format<TYPE>;
     __shared__ __attribute__((aligned(16))) uint8_t raw[GEMV_GN * GEMV_CHUNK * gemv_slot_bytes<TYPE>() + GEMV_CHUNK * 4];

@@ -1382,12 +1382,13 @@ TGO_DEVICE bool gemv_find_task(const GemvArgs & a, int task, int tid, int * shar
 // (every grouped call, every dense call of up to GEMV_ROWS rows) a wave per SIMD if they share the code.
 // FUSED: bf16 activations, quantized by the workgroups themselves (gemv_task), and, for grouped calls, the task looked
 // up in the group list instead of a task list (gemv_find_task): the whole call is this one launch.
-// Three workgroups per CU are asked of the compiler for the fused IQ2_S instances of more than two rows (their eight-row
-// routine alone would take 223 registers and leave room for two): it spills a little in that routine, which few tasks
-// of a decode batch take, and the tasks of one to four rows gain the third workgroup.  The other formats' instances
-// spill three times as much under the same bound and measured slower with it.
+// Three workgroups per CU are asked of the compiler for the instances of more than two rows whose eight-row routine
+// alone would take 180 to 250 registers and leave room for two, where it spills little to get there (IQ2_S 28 and, fused,
+// 116 bytes of scratch per lane, Q5_K 36, Q6_K 52, all inside the routines for five to eight rows, which few tasks of a
+// decode batch take): the tasks of one to four rows gain the third workgroup.  The other instances (Q3_K, the fused
+// Q6_K ones, long rows) spill three times as much under the same bound and measured slower with it; Q4_K fits as it is.
 template <int TYPE, int MAX_ROWS, int FOLD, bool WALK = false, bool FUSED = false>
-__global__ __launch_bounds__(GEMV_THREADS, (FUSED && MAX_ROWS > 2 && TYPE == IQ2_S && FOLD == 1) ? 3 : 1)
+__global__ __launch_bounds__(GEMV_THREADS, (MAX_ROWS > 2 && FOLD == 1 && !WALK && (TYPE == IQ2_S || (!FUSED && (TYPE == Q5_K || TYPE == Q6_K)))) ? 3 : 1)
 void mmq_gemv_kernel(const GemvArgs a) {
     static_assert(!WALK || MAX_ROWS == GEMV_ROWS, "a walked call has full chunks");
     using F = Format<TYPE>;
